@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Headline benchmark: the Qwen3.5-2B-like decode matvec set on one MI355X.
+
+A step is one pass of the decode set at N = 1 token: attention_in [q|k|v], mixer_out
+[o], ffn_in [gate|up] (Q4_K), ffn_down (Q6_K) and the 151,936-row lm_head (Q6_K),
+285.6 MB of packed weights, issued in decode order on one stream as one recorded
+graph.  Inputs and weights are resident in HBM before the timed region.  Steps
+rotate over distinct copies of the weights so that no step finds its weights in the
+256 MB last-level cache.
+
+Prints one JSON line: value = weight bytes per second over the whole set, roofline =
+the dominant kernel (the Q6_K lm_head GEMV) against the 8 TB/s HBM peak, timed live
+with HIP events on the library's stream, and cpu_baseline = the same set on the
+host's cores through the reference's own CPU code (or its C restatement).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+
+import __graft_entry__ as entry
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--lm-head-copies", type=int, default=3)
+    ap.add_argument("--layer-copies", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--details", action="store_true",
+                    help="also time every stage and the other configurations (stderr)")
+    return ap.parse_args()
+
+
+def log(*args):
+    print(*args, file=sys.stderr, flush=True)
+
+
+class DecodeSet:
+    """Device-resident copies of the config-2 matrices and the stage calls."""
+
+    def __init__(self, capi, cfg, synth, layer_copies, head_copies):
+        self.capi, self.cfg = capi, cfg
+        self.host = {name: spec.build() for name, spec in cfg.CONFIG2.items()}
+        self.layers = []
+        for _ in range(layer_copies):
+            self.layers.append({n: capi.Matrix(s.ggml_type, self.host[n], s.rows, s.cols)
+                                for n, s in cfg.CONFIG2.items() if n != "lm_head"})
+        head = cfg.CONFIG2["lm_head"]
+        self.heads = [capi.Matrix(head.ggml_type, self.host["lm_head"], head.rows, head.cols)
+                      for _ in range(head_copies)]
+        self.x_host = synth.activations(1, cfg.HIDDEN2, cfg.CONFIG2_X_SEED)
+        self.act_host = synth.activations(1, cfg.FFN2, cfg.CONFIG2_ACT_SEED)
+        self.x = capi.DeviceBuffer.from_array(self.x_host)
+        self.act = capi.DeviceBuffer.from_array(self.act_host)
+        self.out = {stage: capi.DeviceBuffer(4 * sum(cfg.CONFIG2[n].rows for n in names))
+                    for stage, names in cfg.CONFIG2_STAGES.items()}
+
+    def stage(self, stage, copy):
+        capi, cfg = self.capi, self.cfg
+        if stage == "lm_head":
+            mats = [self.heads[copy % len(self.heads)]]
+        else:
+            layer = self.layers[copy % len(self.layers)]
+            mats = [layer[n] for n in cfg.CONFIG2_STAGES[stage]]
+        x = self.act if stage == "ffn_down" else self.x
+        capi.gemv_dev([capi.whole(m) for m in mats], x, 1, self.out[stage])
+
+    def step(self, copy):
+        for stage in self.cfg.CONFIG2_STAGES:
+            self.stage(stage, copy)
+
+    def record(self, copy):
+        self.capi.capture_begin()
+        self.step(copy)
+        return self.capi.capture_end()
+
+
+def time_graphs(capi, graphs, steps, warmup):
+    for i in range(warmup):
+        graphs[i % len(graphs)].launch()
+    capi.synchronize()
+    capi.timer_begin()
+    for i in range(steps):
+        graphs[(warmup + i) % len(graphs)].launch()
+    ms = capi.timer_end()
+    capi.synchronize()
+    return ms / steps
+
+
+def time_calls(capi, call, steps, warmup):
+    for i in range(warmup):
+        call(i)
+    capi.synchronize()
+    capi.timer_begin()
+    for i in range(steps):
+        call(warmup + i)
+    ms = capi.timer_end()
+    capi.synchronize()
+    return ms / steps
+
+
+def cpu_baseline(cfg, decode, seconds):
+    """The same set on the host cores: the reference's fused AVX2 dots on its own
+    thread pool (oracle/_ref), or the scalar C restatement where that is absent."""
+    oracle = entry.load_oracle()
+    use_ref = oracle.ref_available()
+    if use_ref:
+        threads = oracle.ref().ref_default_threads()
+        kind = "reference"
+    else:
+        import os
+        threads = max(len(os.sched_getaffinity(0)) // 2, 1)
+        kind = "port"
+    stages = []
+    for stage, names in cfg.CONFIG2_STAGES.items():
+        parts = [(cfg.CONFIG2[n].ggml_type, decode.host[n], 0, cfg.CONFIG2[n].rows)
+                 for n in names]
+        stages.append((parts, decode.act_host if stage == "ffn_down" else decode.x_host))
+
+    def one_set():
+        for parts, x in stages:
+            oracle.matmul(parts, x, threads=threads, use_ref=use_ref)
+
+    one_set()  # warm the pool and the page tables
+    t0 = time.perf_counter()
+    one_set()
+    probe = time.perf_counter() - t0
+    reps = int(max(3, min(400, seconds / max(probe, 1e-6))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        one_set()
+    elapsed = time.perf_counter() - t0
+    per_set = elapsed / reps
+    gbs = cfg.config2_bytes() / per_set / 1e9
+    what = ("gguf_dot AVX2 dots on the reference's SpinPool" if use_ref
+            else "scalar C restatement, pthreads")
+    return {"value": round(gbs, 3), "unit": "GB/s", "cores": threads, "kind": kind,
+            "sample": f"{reps} passes of the full 285.6 MB decode set ({what}), "
+                      f"{per_set * 1e3:.2f} ms per set"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only; rerun with --gpus 1 "
+              "(each box has one GPU and the path needs no collective)", file=sys.stderr)
+        sys.exit(2)
+    entry.load_package()
+    from gufo_npu_amd import capi, configs as cfg, synth
+
+    capi.init(0)
+    device, cus = capi.device_info()
+    log(f"device: {device}, {cus} CUs")
+    t0 = time.perf_counter()
+    decode = DecodeSet(capi, cfg, synth, args.layer_copies, args.lm_head_copies)
+    log(f"weights resident: {args.layer_copies} layer copies, {args.lm_head_copies} "
+        f"lm_head copies ({time.perf_counter() - t0:.1f} s)")
+
+    set_bytes = cfg.config2_bytes()
+    n_graphs = max(args.layer_copies, args.lm_head_copies)
+    n_graphs = args.layer_copies * args.lm_head_copies // np.gcd(args.layer_copies,
+                                                                 args.lm_head_copies)
+    n_graphs = min(n_graphs, 30)
+    decode.step(0)
+    capi.synchronize()
+    graphs = [decode.record(i) for i in range(n_graphs)]
+
+    # The timed region: exactly `steps` decode sets after `warmup` untimed ones.
+    capi.synchronize()
+    ms_step = time_graphs(capi, graphs, args.steps, args.warmup)
+    value = set_bytes / (ms_step * 1e-3) / 1e9
+
+    # Dominant kernel: the lm_head GEMV, back to back over the rotating copies.
+    head = cfg.CONFIG2["lm_head"]
+    head_bytes = head.nbytes + 4 * (head.cols + head.rows)
+    ms_head = time_calls(capi, lambda i: decode.stage("lm_head", i), args.steps, args.warmup)
+    achieved = head_bytes / (ms_head * 1e-3) / 1e9
+
+    result = {
+        "metric": "K-quant GEMV HBM GB/s (% of peak) + µs per decode-token matvec set, 1 GPU",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Qwen3.5-2B-like decode matvec set, N=1: q 2048x2048, k/v 512x2048, "
+                        "o 2048x2048, gate/up 6144x2048 (Q4_K), down 2048x6144 (Q6_K), "
+                        "lm_head 151936x2048 (Q6_K); x fp32 N(0,1)",
+            "weight_bytes_per_step": set_bytes,
+            "us_per_set": round(ms_step * 1e3, 3),
+            "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+            "launches_per_step": len(cfg.CONFIG2_STAGES),
+            "weight_copies": {"layer": args.layer_copies, "lm_head": args.lm_head_copies},
+            "device": device,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "KquantGemvKernel<Q6_K, N=1> (lm_head 151936x2048)",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(ms_head * 1e3, 3),
+            "bytes_per_launch": head_bytes,
+            "traffic": None,
+        },
+    }
+
+    if args.details:
+        for stage, names in cfg.CONFIG2_STAGES.items():
+            nbytes = sum(cfg.CONFIG2[n].nbytes for n in names)
+            ms = time_calls(capi, lambda i, s=stage: decode.stage(s, i), args.steps, args.warmup)
+            log(f"  {stage:13s} {nbytes / 1e6:8.2f} MB  {ms * 1e3:8.2f} us  "
+                f"{nbytes / ms / 1e6:8.1f} GB/s")
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg, decode, args.cpu_seconds)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result, ensure_ascii=False))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,117 @@
+// Small kernels beside the matrix products: the greedy pick over logits and a
+// streaming-read probe that measures the read bandwidth a kernel can reach.
+#include "kernels.hpp"
+#include "kquant_common.hpp"
+
+namespace gufo {
+namespace {
+
+struct Best {
+  float value;
+  uint32_t index;
+};
+
+// The better of two candidates under std::max_element's rule (first maximum
+// wins): the larger value, the lower index on equal values
+// (src/core/sampling.cpp:327-329 of the reference).
+__device__ __forceinline__ Best Better(Best a, Best b) {
+  const bool take_b = b.value > a.value || (b.value == a.value && b.index < a.index);
+  return take_b ? b : a;
+}
+
+__device__ __forceinline__ Best WaveBest(Best v) {
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o;
+    o.value = __shfl_xor(v.value, off, 64);
+    o.index = __shfl_xor(v.index, off, 64);
+    v = Better(v, o);
+  }
+  return v;
+}
+
+__device__ __forceinline__ Best BlockBest(Best v) {
+  __shared__ Best per_wave[4];
+  v = WaveBest(v);
+  if ((threadIdx.x & 63) == 0) per_wave[threadIdx.x >> 6] = v;
+  __syncthreads();
+  Best r = per_wave[0];
+  for (int w = 1; w < 4; ++w) r = Better(r, per_wave[w]);
+  return r;
+}
+
+__global__ __launch_bounds__(256) void ArgmaxPartial(const float* __restrict__ v,
+                                                     uint32_t n, Best* partial) {
+  Best best;
+  best.value = -INFINITY;
+  best.index = 0xFFFFFFFFu;
+  for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    Best c;
+    c.value = v[i];
+    c.index = i;
+    best = Better(best, c);
+  }
+  best = BlockBest(best);
+  if (threadIdx.x == 0) partial[blockIdx.x] = best;
+}
+
+__global__ __launch_bounds__(256) void ArgmaxFinal(const Best* partial, uint32_t count,
+                                                   int64_t* out) {
+  Best best;
+  best.value = -INFINITY;
+  best.index = 0xFFFFFFFFu;
+  for (uint32_t i = threadIdx.x; i < count; i += 256) best = Better(best, partial[i]);
+  best = BlockBest(best);
+  if (threadIdx.x == 0) {
+    // All -inf (or NaN) input: max_element returns the first element.
+    *out = best.index == 0xFFFFFFFFu ? 0 : static_cast<int64_t>(best.index);
+  }
+}
+
+__global__ __launch_bounds__(256) void ReadProbe(const U32x4* __restrict__ src,
+                                                 size_t n_vec, uint32_t* sink) {
+  uint32_t acc = 0;
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  // Four independent 16-byte loads in flight per lane.
+  for (; i + 3 * stride < n_vec; i += 4 * stride) {
+    const U32x4 a = __builtin_nontemporal_load(src + i);
+    const U32x4 b = __builtin_nontemporal_load(src + i + stride);
+    const U32x4 c = __builtin_nontemporal_load(src + i + 2 * stride);
+    const U32x4 d = __builtin_nontemporal_load(src + i + 3 * stride);
+    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
+    acc ^= c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  }
+  for (; i < n_vec; i += stride) {
+    const U32x4 a = src[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+  for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, 64);
+  if ((threadIdx.x & 63) == 0) atomicXor(sink, acc);
+}
+
+}  // namespace
+
+hipError_t LaunchArgmax(const float* v, size_t n, void* scratch, int64_t* out,
+                        hipStream_t stream) {
+  if (n == 0 || n > 0xFFFFFFF0ull) return hipErrorInvalidValue;
+  Best* partial = static_cast<Best*>(scratch);
+  uint32_t blocks = static_cast<uint32_t>((n + 1023) / 1024);
+  if (blocks > static_cast<uint32_t>(kArgmaxBlocks)) blocks = kArgmaxBlocks;
+  hipLaunchKernelGGL(ArgmaxPartial, dim3(blocks), dim3(256), 0, stream, v,
+                     static_cast<uint32_t>(n), partial);
+  hipLaunchKernelGGL(ArgmaxFinal, dim3(1), dim3(256), 0, stream, partial, blocks, out);
+  return hipGetLastError();
+}
+
+hipError_t LaunchReadProbe(const void* src, size_t bytes, uint32_t* sink,
+                           hipStream_t stream) {
+  const size_t n_vec = bytes / 16;
+  if (n_vec == 0) return hipSuccess;
+  size_t blocks = (n_vec + 256 * 4 - 1) / (256 * 4);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL(ReadProbe, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+                     stream, static_cast<const U32x4*>(src), n_vec, sink);
+  return hipGetLastError();
+}
+
+}  // namespace gufo

@@ -1,0 +1,865 @@
+// The C-ABI of include/gufo_hip.h: argument checks, device residency of the
+// matrices, launch planning and the one stream every call is ordered on.
+#include "../../include/gufo_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+
+#include "kernels.hpp"
+#include "kquant_common.hpp"
+
+struct gufo_hip_matrix {
+  int type;
+  size_t rows;
+  size_t cols;
+  size_t row_bytes;
+  size_t bytes;
+  uint8_t* data;  // device
+};
+
+struct gufo_hip_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+
+namespace {
+
+using gufo::GemvLaunch;
+using gufo::kMaxGemvParts;
+using gufo::kMaxGemvTokens;
+
+thread_local std::string t_error;
+
+int Fail(int code, const char* format, ...) {
+  char text[512];
+  va_list args;
+  va_start(args, format);
+  std::vsnprintf(text, sizeof text, format, args);
+  va_end(args);
+  t_error = text;
+  return code;
+}
+
+// A device allocation that only grows.  Growing waits for the stream first: work
+// in flight may still use the old block.
+struct Scratch {
+  void* ptr = nullptr;
+  size_t capacity = 0;
+};
+
+struct State {
+  std::mutex mutex;
+  bool ready = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+  hipEvent_t timer_begin = nullptr;
+  hipEvent_t timer_end = nullptr;
+  char name[256] = {0};
+  int compute_units = 0;
+  long live_matrices = 0;
+  bool moe_pending = false;  // an expert call since the last synchronize
+  bool capturing = false;    // between capture_begin and capture_end
+  Scratch small;             // argmax partials + result, MoE tables header
+  Scratch stage_x;           // host-pointer variants: device copies of x, y, ...
+  Scratch stage_y;
+  Scratch stage_ids;
+  Scratch stage_weights;
+  Scratch moe_tables;   // counts, offsets, pairs, valid flags, segments
+  Scratch moe_gate_up;  // pairs x 2*ffn
+  Scratch moe_out;      // pairs x hidden
+};
+
+State g_state;
+
+#define GUFO_HIP_TRY(expr)                                                        \
+  do {                                                                            \
+    const hipError_t gufo_status_ = (expr);                                       \
+    if (gufo_status_ != hipSuccess) {                                             \
+      return Fail(gufo_status_ == hipErrorOutOfMemory ? GUFO_HIP_ERR_OUT_OF_MEMORY \
+                                                      : GUFO_HIP_ERR_RUNTIME,     \
+                  "%s: %s", #expr, hipGetErrorString(gufo_status_));              \
+    }                                                                             \
+  } while (0)
+
+#define GUFO_TRY(expr)                      \
+  do {                                      \
+    const int gufo_code_ = (expr);          \
+    if (gufo_code_ != GUFO_HIP_OK) return gufo_code_; \
+  } while (0)
+
+int RequireReady() {
+  if (!g_state.ready) {
+    return Fail(GUFO_HIP_ERR_NOT_INITIALIZED, "gufo_hip_init has not been called");
+  }
+  return GUFO_HIP_OK;
+}
+
+int Reserve(Scratch* s, size_t bytes) {
+  if (bytes <= s->capacity) return GUFO_HIP_OK;
+  if (g_state.capturing) {
+    return Fail(GUFO_HIP_ERR_LOGIC,
+                "a recorded call needs %zu bytes of scratch; make the same call once "
+                "before recording",
+                bytes);
+  }
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  if (s->ptr != nullptr) {
+    GUFO_HIP_TRY(hipFree(s->ptr));
+    s->ptr = nullptr;
+    s->capacity = 0;
+  }
+  const size_t rounded = (bytes + 0xFFFFu) & ~static_cast<size_t>(0xFFFFu);
+  GUFO_HIP_TRY(hipMalloc(&s->ptr, rounded));
+  s->capacity = rounded;
+  return GUFO_HIP_OK;
+}
+
+void Release(Scratch* s) {
+  if (s->ptr != nullptr) (void)hipFree(s->ptr);
+  s->ptr = nullptr;
+  s->capacity = 0;
+}
+
+// Layout of State::small.
+constexpr size_t kArgmaxPartialBytes = static_cast<size_t>(gufo::kArgmaxBlocks) * 8;
+constexpr size_t kArgmaxResultOffset = kArgmaxPartialBytes;
+constexpr size_t kMoeHeaderOffset = kArgmaxResultOffset + 64;
+constexpr size_t kSmallBytes = kMoeHeaderOffset + 64;
+
+// Device addresses of the grouping tables inside State::moe_tables.
+struct MoeTablePointers {
+  int* counts;
+  int* offsets;
+  int* pairs;
+  uint8_t* valid;
+  gufo::MoeSegment* segments;
+  gufo::MoeTables* header;
+};
+
+size_t Align16(size_t v) { return (v + 15) & ~static_cast<size_t>(15); }
+
+int ReserveMoeTables(int n_pairs, int experts, MoeTablePointers* out) {
+  const size_t counts_bytes = Align16(sizeof(int) * static_cast<size_t>(experts));
+  const size_t offsets_bytes = Align16(sizeof(int) * (static_cast<size_t>(experts) + 1));
+  const size_t pairs_bytes = Align16(sizeof(int) * static_cast<size_t>(n_pairs));
+  const size_t valid_bytes = Align16(static_cast<size_t>(n_pairs));
+  const size_t segment_bytes =
+      Align16(sizeof(gufo::MoeSegment) * static_cast<size_t>(n_pairs));
+  GUFO_TRY(Reserve(&g_state.moe_tables, counts_bytes + offsets_bytes + pairs_bytes +
+                                            valid_bytes + segment_bytes + 16));
+  uint8_t* base = static_cast<uint8_t*>(g_state.moe_tables.ptr);
+  out->counts = reinterpret_cast<int*>(base);
+  base += counts_bytes;
+  out->offsets = reinterpret_cast<int*>(base);
+  base += offsets_bytes;
+  out->pairs = reinterpret_cast<int*>(base);
+  base += pairs_bytes;
+  out->valid = base;
+  base += valid_bytes;
+  out->segments = reinterpret_cast<gufo::MoeSegment*>(base);
+  out->header = reinterpret_cast<gufo::MoeTables*>(
+      static_cast<uint8_t*>(g_state.small.ptr) + kMoeHeaderOffset);
+  return GUFO_HIP_OK;
+}
+
+bool Aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The checks GgufProjections makes when it is built and when a stage is applied
+// (src/models/qwen35/gguf_projections.cpp:27-46,213-215 of the reference).
+int CheckParts(const gufo_hip_matrix* const* parts, const size_t* first_row,
+               const size_t* n_rows, int n_parts, int tokens, size_t* stride) {
+  if (n_parts <= 0 || parts == nullptr || first_row == nullptr || n_rows == nullptr) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product (n_parts = %d)", n_parts);
+  }
+  if (tokens < 0) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "tokens = %d", tokens);
+  size_t total = 0;
+  for (int p = 0; p < n_parts; ++p) {
+    if (parts[p] == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "part %d has no matrix", p);
+    if (parts[p]->cols != parts[0]->cols) {
+      return Fail(GUFO_HIP_ERR_SHAPE,
+                  "part %d has %zu columns, expected %zu: parts of one product share "
+                  "their input",
+                  p, parts[p]->cols, parts[0]->cols);
+    }
+    if (first_row[p] > parts[p]->rows || n_rows[p] > parts[p]->rows - first_row[p]) {
+      return Fail(GUFO_HIP_ERR_OUT_OF_RANGE,
+                  "part %d: rows [%zu, %zu) of a matrix with %zu rows", p, first_row[p],
+                  first_row[p] + n_rows[p], parts[p]->rows);
+    }
+    total += n_rows[p];
+  }
+  if (total > 0xFFFFFFF0ull) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu output rows exceed the launch limit",
+                total);
+  }
+  *stride = total;
+  return GUFO_HIP_OK;
+}
+
+int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                  const size_t* n_rows, int n_parts, const float* x, int tokens,
+                  float* y) {
+  size_t stride = 0;
+  GUFO_TRY(CheckParts(parts, first_row, n_rows, n_parts, tokens, &stride));
+  if (tokens == 0 || stride == 0) return GUFO_HIP_OK;
+  if (x == nullptr || y == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x or y is null");
+  }
+  if (!Aligned16(x)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
+  }
+  const size_t cols = parts[0]->cols;
+  for (int t0 = 0; t0 < tokens; t0 += kMaxGemvTokens) {
+    const int nt = tokens - t0 < kMaxGemvTokens ? tokens - t0 : kMaxGemvTokens;
+    size_t offset = 0;
+    int p = 0;
+    while (p < n_parts) {
+      // One launch per run of parts of one type.
+      GemvLaunch launch;
+      std::memset(&launch, 0, sizeof launch);
+      const int type = parts[p]->type;
+      uint32_t total = 0;
+      uint32_t count = 0;
+      while (p < n_parts && parts[p]->type == type &&
+             count < static_cast<uint32_t>(kMaxGemvParts)) {
+        launch.part[count].rows = parts[p]->data + first_row[p] * parts[p]->row_bytes;
+        launch.part[count].n_rows = static_cast<uint32_t>(n_rows[p]);
+        launch.part[count].y_offset = static_cast<uint32_t>(offset);
+        offset += n_rows[p];
+        total += static_cast<uint32_t>(n_rows[p]);
+        ++count;
+        ++p;
+      }
+      launch.n_parts = count;
+      launch.total_rows = total;
+      launch.blocks_per_row = static_cast<uint32_t>(cols / gufo::kSuperBlock);
+      launch.y_stride = static_cast<uint32_t>(stride);
+      GUFO_HIP_TRY(gufo::LaunchGemv(type, launch, x + static_cast<size_t>(t0) * cols, nt,
+                                    y + static_cast<size_t>(t0) * stride,
+                                    g_state.stream));
+    }
+  }
+  return GUFO_HIP_OK;
+}
+
+int CopyIn(Scratch* stage, const void* host, size_t bytes) {
+  GUFO_TRY(Reserve(stage, bytes > 0 ? bytes : 16));
+  if (bytes > 0) {
+    GUFO_HIP_TRY(hipMemcpyAsync(stage->ptr, host, bytes, hipMemcpyHostToDevice,
+                                g_state.stream));
+  }
+  return GUFO_HIP_OK;
+}
+
+int CopyOut(void* host, const void* device, size_t bytes) {
+  if (bytes > 0) {
+    GUFO_HIP_TRY(hipMemcpyAsync(host, device, bytes, hipMemcpyDeviceToHost,
+                                g_state.stream));
+  }
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int RouteDevLocked(const float* logits, int tokens, int experts, int k, int* ids,
+                   float* weights) {
+  if (tokens < 0 || k <= 0 || experts <= 0 || k > experts) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "route: tokens %d, experts %d, k %d",
+                tokens, experts, k);
+  }
+  if (experts > gufo::kMaxRouteExperts || k > gufo::kMaxRouteK) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "route: at most %d experts and k <= %d are supported",
+                gufo::kMaxRouteExperts, gufo::kMaxRouteK);
+  }
+  if (tokens == 0) return GUFO_HIP_OK;
+  GUFO_HIP_TRY(gufo::LaunchRoute(logits, tokens, experts, k, ids, weights, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int GroupDevLocked(const int* ids, int tokens, int k, int experts,
+                   MoeTablePointers* tables) {
+  if (tokens < 0 || k <= 0 || experts <= 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "group: tokens %d, k %d, experts %d",
+                tokens, k, experts);
+  }
+  const long n_pairs = static_cast<long>(tokens) * k;
+  if (n_pairs > gufo::kMaxGroupPairs || experts > gufo::kMaxGroupExperts) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "group: at most %d (token, slot) pairs and %d experts per call",
+                gufo::kMaxGroupPairs, gufo::kMaxGroupExperts);
+  }
+  GUFO_TRY(ReserveMoeTables(static_cast<int>(n_pairs > 0 ? n_pairs : 1), experts, tables));
+  GUFO_HIP_TRY(gufo::LaunchMoeGroup(ids, static_cast<int>(n_pairs), experts,
+                                    tables->counts, tables->offsets, tables->pairs,
+                                    tables->valid, tables->segments, tables->header,
+                                    g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                    const gufo_hip_matrix* down, int experts, const float* x, int tokens,
+                    const int* ids, const float* weights, int k, float* y) {
+  if (gate == nullptr || up == nullptr || down == nullptr) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no MoE experts");
+  }
+  if (experts <= 0 || tokens < 0 || k <= 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: experts %d, tokens %d, k %d",
+                experts, tokens, k);
+  }
+  const size_t e = static_cast<size_t>(experts);
+  const size_t hidden = gate->cols;
+  if (gate->rows % e != 0 || up->rows != gate->rows || up->cols != hidden ||
+      down->rows != e * hidden || down->cols * e != gate->rows) {
+    return Fail(GUFO_HIP_ERR_SHAPE,
+                "expert tensors gate [%zu x %zu], up [%zu x %zu], down [%zu x %zu] do "
+                "not describe %d experts of one width",
+                gate->rows, gate->cols, up->rows, up->cols, down->rows, down->cols,
+                experts);
+  }
+  const size_t ffn = gate->rows / e;
+  if (tokens == 0) return GUFO_HIP_OK;
+  if (x == nullptr || y == nullptr || ids == nullptr || weights == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: null buffer");
+  }
+  if (!Aligned16(x)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
+  MoeTablePointers tables;
+  GUFO_TRY(GroupDevLocked(ids, tokens, k, experts, &tables));
+  const size_t n_pairs = static_cast<size_t>(tokens) * k;
+  GUFO_TRY(Reserve(&g_state.moe_gate_up, n_pairs * 2 * ffn * sizeof(float)));
+  GUFO_TRY(Reserve(&g_state.moe_out, n_pairs * hidden * sizeof(float)));
+  float* gate_up = static_cast<float*>(g_state.moe_gate_up.ptr);
+  float* routed = static_cast<float*>(g_state.moe_out.ptr);
+
+  gufo::MoeGemvArgs args;
+  std::memset(&args, 0, sizeof args);
+  args.tables = tables.header;
+  args.segments = tables.segments;
+  args.k = static_cast<uint32_t>(k);
+
+  // [gate | up] of every pair: kExpertIn's layout.
+  args.x = x;
+  args.x_row_floats = hidden;
+  args.y = gate_up;
+  const gufo_hip_matrix* in_parts[2] = {gate, up};
+  for (int first = 0; first < 2;) {
+    GemvLaunch launch;
+    std::memset(&launch, 0, sizeof launch);
+    int count = 0;
+    const int type = in_parts[first]->type;
+    for (int p = first; p < 2 && in_parts[p]->type == type; ++p) {
+      launch.part[count].rows = in_parts[p]->data;
+      launch.part[count].n_rows = static_cast<uint32_t>(ffn);
+      launch.part[count].y_offset = static_cast<uint32_t>(p * ffn);
+      args.expert_bytes[count] = ffn * in_parts[p]->row_bytes;
+      ++count;
+    }
+    launch.n_parts = static_cast<uint32_t>(count);
+    launch.total_rows = static_cast<uint32_t>(count * ffn);
+    launch.blocks_per_row = static_cast<uint32_t>(hidden / gufo::kSuperBlock);
+    launch.y_stride = static_cast<uint32_t>(2 * ffn);
+    GUFO_HIP_TRY(gufo::LaunchMoeGemv(type, launch, args, false,
+                                     static_cast<uint32_t>(n_pairs), g_state.stream));
+    first += count;
+  }
+
+  // down over silu(gate) * up of every pair.
+  {
+    GemvLaunch launch;
+    std::memset(&launch, 0, sizeof launch);
+    launch.part[0].rows = down->data;
+    launch.part[0].n_rows = static_cast<uint32_t>(hidden);
+    launch.part[0].y_offset = 0;
+    launch.n_parts = 1;
+    launch.total_rows = static_cast<uint32_t>(hidden);
+    launch.blocks_per_row = static_cast<uint32_t>(ffn / gufo::kSuperBlock);
+    launch.y_stride = static_cast<uint32_t>(hidden);
+    args.x = gate_up;
+    args.x_row_floats = 2 * ffn;
+    args.y = routed;
+    std::memset(args.expert_bytes, 0, sizeof args.expert_bytes);
+    args.expert_bytes[0] = hidden * down->row_bytes;
+    GUFO_HIP_TRY(gufo::LaunchMoeGemv(down->type, launch, args, true,
+                                     static_cast<uint32_t>(n_pairs), g_state.stream));
+  }
+  GUFO_HIP_TRY(gufo::LaunchMoeCombine(routed, weights, tables.valid, tokens, k,
+                                      static_cast<int>(hidden), y, g_state.stream));
+  g_state.moe_pending = true;
+  return GUFO_HIP_OK;
+}
+
+// After a synchronize: were any expert ids of the calls since the last one out of
+// range?  GgufProjections::ApplyExpert throws std::logic_error for those
+// (src/models/qwen35/gguf_projections.cpp:222-224 of the reference).
+int CheckMoeIdsLocked() {
+  if (!g_state.moe_pending) return GUFO_HIP_OK;
+  g_state.moe_pending = false;
+  gufo::MoeTables header;
+  GUFO_HIP_TRY(hipMemcpy(&header,
+                         static_cast<uint8_t*>(g_state.small.ptr) + kMoeHeaderOffset,
+                         sizeof header, hipMemcpyDeviceToHost));
+  if (header.n_invalid != 0) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "no such expert: %d routed ids were out of range",
+                header.n_invalid);
+  }
+  return GUFO_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gufo_hip_init(int device) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  if (g_state.ready) {
+    if (g_state.device == device) return GUFO_HIP_OK;
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "already initialised on device %d; shut down first", g_state.device);
+  }
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return Fail(GUFO_HIP_ERR_NO_DEVICE, "gufo_hip: no HIP device is available");
+  }
+  if (device < 0 || device >= count) {
+    return Fail(GUFO_HIP_ERR_NO_DEVICE, "gufo_hip: device %d of %d does not exist", device,
+                count);
+  }
+  hipDeviceProp_t prop;
+  GUFO_HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    return Fail(GUFO_HIP_ERR_NO_DEVICE,
+                "gufo_hip: device %d is %s; this library is built for gfx950 only", device,
+                prop.gcnArchName);
+  }
+  GUFO_HIP_TRY(hipSetDevice(device));
+  GUFO_HIP_TRY(hipStreamCreateWithFlags(&g_state.stream, hipStreamNonBlocking));
+  GUFO_HIP_TRY(hipEventCreate(&g_state.timer_begin));
+  GUFO_HIP_TRY(hipEventCreate(&g_state.timer_end));
+  std::snprintf(g_state.name, sizeof g_state.name, "%s (%s)", prop.gcnArchName, prop.name);
+  g_state.compute_units = prop.multiProcessorCount;
+  g_state.device = device;
+  g_state.ready = true;
+  const int code = Reserve(&g_state.small, kSmallBytes);
+  if (code != GUFO_HIP_OK) {
+    g_state.ready = false;
+    return code;
+  }
+  GUFO_HIP_TRY(hipMemsetAsync(g_state.small.ptr, 0, kSmallBytes, g_state.stream));
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_shutdown(void) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  if (!g_state.ready) return GUFO_HIP_OK;
+  if (g_state.live_matrices != 0) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "%ld matrices are still alive", g_state.live_matrices);
+  }
+  (void)hipStreamSynchronize(g_state.stream);
+  Release(&g_state.small);
+  Release(&g_state.stage_x);
+  Release(&g_state.stage_y);
+  Release(&g_state.stage_ids);
+  Release(&g_state.stage_weights);
+  Release(&g_state.moe_tables);
+  Release(&g_state.moe_gate_up);
+  Release(&g_state.moe_out);
+  (void)hipEventDestroy(g_state.timer_begin);
+  (void)hipEventDestroy(g_state.timer_end);
+  (void)hipStreamDestroy(g_state.stream);
+  g_state.stream = nullptr;
+  g_state.ready = false;
+  g_state.device = -1;
+  return GUFO_HIP_OK;
+}
+
+const char* gufo_hip_last_error(void) { return t_error.c_str(); }
+
+int gufo_hip_device_info(char* name, size_t name_bytes, int* compute_units) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (name != nullptr && name_bytes > 0) std::snprintf(name, name_bytes, "%s", g_state.name);
+  if (compute_units != nullptr) *compute_units = g_state.compute_units;
+  return GUFO_HIP_OK;
+}
+
+size_t gufo_hip_block_bytes(int ggml_type) {
+  return static_cast<size_t>(gufo::BlockBytes(ggml_type));
+}
+
+size_t gufo_hip_row_bytes(int ggml_type, size_t cols) {
+  const size_t block = gufo_hip_block_bytes(ggml_type);
+  if (block == 0 || cols % gufo::kSuperBlock != 0) return 0;
+  return cols / gufo::kSuperBlock * block;
+}
+
+int gufo_hip_malloc(void** device_ptr, size_t bytes) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (device_ptr == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null out pointer");
+  *device_ptr = nullptr;
+  GUFO_HIP_TRY(hipMalloc(device_ptr, bytes > 0 ? bytes : 16));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_free(void* device_ptr) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (device_ptr == nullptr) return GUFO_HIP_OK;
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  GUFO_HIP_TRY(hipFree(device_ptr));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (bytes == 0) return GUFO_HIP_OK;
+  GUFO_HIP_TRY(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice,
+                              g_state.stream));
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return CopyOut(host_dst, device_src, bytes);
+}
+
+int gufo_hip_synchronize(void) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  return CheckMoeIdsLocked();
+}
+
+int gufo_hip_matrix_create(int ggml_type, const void* host_blocks, size_t rows,
+                           size_t cols, gufo_hip_matrix** out) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (out == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null out pointer");
+  *out = nullptr;
+  if (gufo_hip_block_bytes(ggml_type) == 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "unknown ggml type %d", ggml_type);
+  }
+  const size_t row_bytes = gufo_hip_row_bytes(ggml_type, cols);
+  if (row_bytes == 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "row is not a whole number of blocks (%zu values)", cols);
+  }
+  if (rows > 0xFFFFFFF0ull || cols > (1ull << 24)) {
+    return Fail(GUFO_HIP_ERR_SHAPE, "matrix %zu x %zu exceeds the launch limits", rows, cols);
+  }
+  if (host_blocks == nullptr && rows != 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null weight data");
+  }
+  gufo_hip_matrix* m = new (std::nothrow) gufo_hip_matrix;
+  if (m == nullptr) return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "host allocation failed");
+  m->type = ggml_type;
+  m->rows = rows;
+  m->cols = cols;
+  m->row_bytes = row_bytes;
+  m->bytes = rows * row_bytes;
+  m->data = nullptr;
+  // 64 spare bytes: the last lanes of a wave may prefetch past the final block.
+  const hipError_t status =
+      hipMalloc(reinterpret_cast<void**>(&m->data), m->bytes + 64);
+  if (status != hipSuccess) {
+    delete m;
+    return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "hipMalloc of %zu bytes: %s", rows * row_bytes,
+                hipGetErrorString(status));
+  }
+  hipError_t copy = hipSuccess;
+  if (m->bytes > 0) {
+    copy = hipMemcpyAsync(m->data, host_blocks, m->bytes, hipMemcpyHostToDevice,
+                          g_state.stream);
+  }
+  if (copy == hipSuccess) {
+    copy = hipMemsetAsync(m->data + m->bytes, 0, 64, g_state.stream);
+  }
+  if (copy == hipSuccess) copy = hipStreamSynchronize(g_state.stream);
+  if (copy != hipSuccess) {
+    (void)hipFree(m->data);
+    delete m;
+    return Fail(GUFO_HIP_ERR_RUNTIME, "upload of the matrix: %s", hipGetErrorString(copy));
+  }
+  ++g_state.live_matrices;
+  *out = m;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_matrix_destroy(gufo_hip_matrix* m) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  if (m == nullptr) return GUFO_HIP_OK;
+  GUFO_TRY(RequireReady());
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  GUFO_HIP_TRY(hipFree(m->data));
+  delete m;
+  --g_state.live_matrices;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_matrix_info(const gufo_hip_matrix* m, int* ggml_type, size_t* rows,
+                         size_t* cols, size_t* bytes) {
+  if (m == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null matrix");
+  if (ggml_type != nullptr) *ggml_type = m->type;
+  if (rows != nullptr) *rows = m->rows;
+  if (cols != nullptr) *cols = m->cols;
+  if (bytes != nullptr) *bytes = m->bytes;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_gemv_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                      const size_t* n_rows, int n_parts, const float* x_dev, int tokens,
+                      float* y_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemvDevLocked(parts, first_row, n_rows, n_parts, x_dev, tokens, y_dev);
+}
+
+int gufo_hip_gemv(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                  const size_t* n_rows, int n_parts, const float* x_host, int tokens,
+                  float* y_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  size_t stride = 0;
+  GUFO_TRY(CheckParts(parts, first_row, n_rows, n_parts, tokens, &stride));
+  if (tokens == 0 || stride == 0) return GUFO_HIP_OK;
+  if (x_host == nullptr || y_host == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x or y is null");
+  }
+  const size_t x_bytes = static_cast<size_t>(tokens) * parts[0]->cols * sizeof(float);
+  const size_t y_bytes = static_cast<size_t>(tokens) * stride * sizeof(float);
+  GUFO_TRY(CopyIn(&g_state.stage_x, x_host, x_bytes));
+  GUFO_TRY(Reserve(&g_state.stage_y, y_bytes));
+  GUFO_TRY(GemvDevLocked(parts, first_row, n_rows, n_parts,
+                         static_cast<const float*>(g_state.stage_x.ptr), tokens,
+                         static_cast<float*>(g_state.stage_y.ptr)));
+  return CopyOut(y_host, g_state.stage_y.ptr, y_bytes);
+}
+
+int gufo_hip_argmax_dev(const float* logits_dev, size_t n, int64_t* index_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (logits_dev == nullptr || index_host == nullptr || n == 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "argmax: empty input");
+  }
+  uint8_t* small = static_cast<uint8_t*>(g_state.small.ptr);
+  int64_t* result = reinterpret_cast<int64_t*>(small + kArgmaxResultOffset);
+  GUFO_HIP_TRY(gufo::LaunchArgmax(logits_dev, n, small, result, g_state.stream));
+  return CopyOut(index_host, result, sizeof(int64_t));
+}
+
+int gufo_hip_route_topk_dev(const float* logits_dev, int tokens, int experts, int k,
+                            int* ids_dev, float* weights_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return RouteDevLocked(logits_dev, tokens, experts, k, ids_dev, weights_dev);
+}
+
+int gufo_hip_route_topk(const float* logits_host, int tokens, int experts, int k,
+                        int* ids_host, float* weights_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (tokens < 0 || k <= 0 || experts <= 0 || k > experts) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "route: tokens %d, experts %d, k %d",
+                tokens, experts, k);
+  }
+  if (tokens == 0) return GUFO_HIP_OK;
+  const size_t n = static_cast<size_t>(tokens) * k;
+  GUFO_TRY(CopyIn(&g_state.stage_x, logits_host,
+                  static_cast<size_t>(tokens) * experts * sizeof(float)));
+  GUFO_TRY(Reserve(&g_state.stage_ids, n * sizeof(int)));
+  GUFO_TRY(Reserve(&g_state.stage_weights, n * sizeof(float)));
+  GUFO_TRY(RouteDevLocked(static_cast<const float*>(g_state.stage_x.ptr), tokens, experts,
+                          k, static_cast<int*>(g_state.stage_ids.ptr),
+                          static_cast<float*>(g_state.stage_weights.ptr)));
+  GUFO_TRY(CopyOut(ids_host, g_state.stage_ids.ptr, n * sizeof(int)));
+  return CopyOut(weights_host, g_state.stage_weights.ptr, n * sizeof(float));
+}
+
+int gufo_hip_moe_group(const int* ids_host, int tokens, int k, int experts,
+                       int* counts_host, int* offsets_host, int* pairs_host,
+                       int* distinct_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (tokens < 0 || k <= 0 || experts <= 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "group: tokens %d, k %d, experts %d",
+                tokens, k, experts);
+  }
+  const size_t n = static_cast<size_t>(tokens) * k;
+  GUFO_TRY(CopyIn(&g_state.stage_ids, ids_host, n * sizeof(int)));
+  MoeTablePointers tables;
+  GUFO_TRY(GroupDevLocked(static_cast<const int*>(g_state.stage_ids.ptr), tokens, k,
+                          experts, &tables));
+  gufo::MoeTables header;
+  GUFO_TRY(CopyOut(&header, tables.header, sizeof header));
+  if (header.n_invalid != 0) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "no such expert: %d routed ids were out of range",
+                header.n_invalid);
+  }
+  if (counts_host != nullptr) {
+    GUFO_TRY(CopyOut(counts_host, tables.counts, sizeof(int) * experts));
+  }
+  if (offsets_host != nullptr) {
+    GUFO_TRY(CopyOut(offsets_host, tables.offsets, sizeof(int) * (experts + 1)));
+  }
+  if (pairs_host != nullptr) GUFO_TRY(CopyOut(pairs_host, tables.pairs, sizeof(int) * n));
+  if (distinct_host != nullptr) *distinct_host = header.n_distinct;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                         const gufo_hip_matrix* down, int experts, const float* x_dev,
+                         int tokens, const int* ids_dev, const float* weights_dev, int k,
+                         float* y_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return MoeFfnDevLocked(gate, up, down, experts, x_dev, tokens, ids_dev, weights_dev, k,
+                         y_dev);
+}
+
+int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                     const gufo_hip_matrix* down, int experts, const float* x_host,
+                     int tokens, const int* ids_host, const float* weights_host, int k,
+                     float* y_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (gate == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no MoE experts");
+  if (tokens < 0 || k <= 0) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: tokens %d, k %d", tokens, k);
+  }
+  if (tokens == 0) return GUFO_HIP_OK;
+  const size_t n = static_cast<size_t>(tokens) * k;
+  const size_t hidden = gate->cols;
+  for (size_t i = 0; i < n; ++i) {
+    if (ids_host[i] < 0 || ids_host[i] >= experts) {
+      return Fail(GUFO_HIP_ERR_LOGIC, "no such expert: %d", ids_host[i]);
+    }
+  }
+  GUFO_TRY(CopyIn(&g_state.stage_x, x_host, tokens * hidden * sizeof(float)));
+  GUFO_TRY(CopyIn(&g_state.stage_ids, ids_host, n * sizeof(int)));
+  GUFO_TRY(CopyIn(&g_state.stage_weights, weights_host, n * sizeof(float)));
+  GUFO_TRY(Reserve(&g_state.stage_y, tokens * hidden * sizeof(float)));
+  GUFO_TRY(MoeFfnDevLocked(gate, up, down, experts,
+                           static_cast<const float*>(g_state.stage_x.ptr), tokens,
+                           static_cast<const int*>(g_state.stage_ids.ptr),
+                           static_cast<const float*>(g_state.stage_weights.ptr), k,
+                           static_cast<float*>(g_state.stage_y.ptr)));
+  GUFO_TRY(CopyOut(y_host, g_state.stage_y.ptr, tokens * hidden * sizeof(float)));
+  return CheckMoeIdsLocked();
+}
+
+int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
+                               size_t m, float* c_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  (void)w;
+  (void)a_bf16_dev;
+  (void)m;
+  (void)c_dev;
+  return Fail(GUFO_HIP_ERR_RUNTIME, "the prefill GEMM is not built into this library yet");
+}
+
+int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
+                           float* c_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  (void)w;
+  (void)a_bf16_host;
+  (void)m;
+  (void)c_host;
+  return Fail(GUFO_HIP_ERR_RUNTIME, "the prefill GEMM is not built into this library yet");
+}
+
+int gufo_hip_capture_begin(void) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (g_state.capturing) return Fail(GUFO_HIP_ERR_LOGIC, "already recording");
+  GUFO_HIP_TRY(hipStreamBeginCapture(g_state.stream, hipStreamCaptureModeThreadLocal));
+  g_state.capturing = true;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_capture_end(gufo_hip_graph** out) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (out == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null out pointer");
+  *out = nullptr;
+  if (!g_state.capturing) return Fail(GUFO_HIP_ERR_LOGIC, "not recording");
+  g_state.capturing = false;
+  hipGraph_t graph = nullptr;
+  GUFO_HIP_TRY(hipStreamEndCapture(g_state.stream, &graph));
+  hipGraphExec_t exec = nullptr;
+  const hipError_t status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (status != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return Fail(GUFO_HIP_ERR_RUNTIME, "hipGraphInstantiate: %s", hipGetErrorString(status));
+  }
+  gufo_hip_graph* g = new (std::nothrow) gufo_hip_graph;
+  if (g == nullptr) {
+    (void)hipGraphExecDestroy(exec);
+    (void)hipGraphDestroy(graph);
+    return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "host allocation failed");
+  }
+  g->graph = graph;
+  g->exec = exec;
+  *out = g;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_graph_launch(gufo_hip_graph* graph) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (graph == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null graph");
+  if (g_state.capturing) return Fail(GUFO_HIP_ERR_LOGIC, "a graph cannot be launched while recording");
+  GUFO_HIP_TRY(hipGraphLaunch(graph->exec, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_graph_destroy(gufo_hip_graph* graph) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  if (graph == nullptr) return GUFO_HIP_OK;
+  GUFO_TRY(RequireReady());
+  GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  (void)hipGraphExecDestroy(graph->exec);
+  (void)hipGraphDestroy(graph->graph);
+  delete graph;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_timer_begin(void) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  GUFO_HIP_TRY(hipEventRecord(g_state.timer_begin, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_timer_end(float* milliseconds) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (milliseconds == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null out pointer");
+  GUFO_HIP_TRY(hipEventRecord(g_state.timer_end, g_state.stream));
+  GUFO_HIP_TRY(hipEventSynchronize(g_state.timer_end));
+  GUFO_HIP_TRY(hipEventElapsedTime(milliseconds, g_state.timer_begin, g_state.timer_end));
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_read_probe_dev(const void* src_dev, size_t bytes, uint32_t* sink_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (src_dev == nullptr || sink_dev == nullptr || !Aligned16(src_dev)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "read probe: null or unaligned buffer");
+  }
+  GUFO_HIP_TRY(gufo::LaunchReadProbe(src_dev, bytes, sink_dev, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+// Internal interface between the C-ABI layer (capi.hip) and the kernel files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace gufo {
+
+constexpr int kMaxGemvParts = 8;   // row ranges per launch
+constexpr int kMaxGemvTokens = 4;  // token columns per pass over the weights
+
+// One row range of a launch: `rows` points at the first byte of its first row.
+struct GemvPart {
+  const uint8_t* rows;
+  uint32_t n_rows;
+  uint32_t y_offset;  // column of the range's first output within a y row
+};
+
+struct GemvLaunch {
+  GemvPart part[kMaxGemvParts];
+  uint32_t n_parts;
+  uint32_t total_rows;      // sum of n_rows
+  uint32_t blocks_per_row;  // cols / 256
+  uint32_t y_stride;        // floats between token rows of y
+};
+
+// y[t*y_stride + part.y_offset + r] = row r of part . x[t*cols ...], t < tokens.
+// All parts are of `type`.  tokens in 1..kMaxGemvTokens.
+hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
+                      float* y, hipStream_t stream);
+
+// ---- mixture of experts ------------------------------------------------------
+
+// One routed expert and up to four of the (token, slot) pairs that chose it.
+// pair = token * k + slot.
+struct MoeSegment {
+  int32_t expert;
+  int32_t n_pairs;
+  int32_t pair[kMaxGemvTokens];
+};
+
+// Written by the grouping kernel, read by the expert kernels.
+struct MoeTables {
+  int32_t n_segments;
+  int32_t n_distinct;  // experts chosen by at least one pair
+  int32_t n_invalid;   // pairs whose expert id is out of range (dropped)
+  int32_t pad;
+};
+
+struct MoeGemvArgs {
+  const MoeTables* tables;
+  const MoeSegment* segments;
+  const float* x;       // activation rows
+  size_t x_row_floats;  // floats between activation rows
+  float* y;             // output rows, one per pair, y_stride floats apart
+  uint32_t k;           // slots per token
+  size_t expert_bytes[kMaxGemvParts];  // bytes between experts, per part
+};
+
+// As LaunchGemv, once per segment: part p's rows start at
+// part[p].rows + segment.expert * expert_bytes[p].  swiglu = false: column t reads
+// x row (pair / k); swiglu = true: column t reads the pair's own row of 2*cols
+// values [gate | up] and the product is taken with silu(gate) * up.
+hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& moe,
+                         bool swiglu, uint32_t max_segments, hipStream_t stream);
+
+// Softmax (double) top-k routing of `tokens` rows of `experts` logits.
+constexpr int kMaxRouteExperts = 1024;
+constexpr int kMaxRouteK = 64;
+hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int* ids,
+                       float* weights, hipStream_t stream);
+
+// Groups the n_pairs = tokens*k pairs by expert: counts[experts],
+// offsets[experts+1], pairs[n_pairs] (ascending pair id within an expert),
+// pair_valid[n_pairs], the segment list (at most n_pairs entries) and *tables.
+constexpr int kMaxGroupExperts = 1024;
+constexpr int kMaxGroupPairs = 8192;
+hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int* counts,
+                          int* offsets, int* pairs, uint8_t* pair_valid,
+                          MoeSegment* segments, MoeTables* tables, hipStream_t stream);
+
+// y[t][i] = sum over slots in order of weights[t*k+slot] * rows[(t*k+slot)][i],
+// accumulated in double; invalid pairs are skipped.
+hipError_t LaunchMoeCombine(const float* rows, const float* weights,
+                            const uint8_t* pair_valid, int tokens, int k, int hidden,
+                            float* y, hipStream_t stream);
+
+// index of the first maximum of v[0..n) -> *out (device); scratch holds
+// 2*kArgmaxBlocks entries of 8 bytes.
+constexpr int kArgmaxBlocks = 1024;
+hipError_t LaunchArgmax(const float* v, size_t n, void* scratch, int64_t* out,
+                        hipStream_t stream);
+
+// Streaming read of `bytes` (multiple of 16) -> xor of all dwords into *sink.
+hipError_t LaunchReadProbe(const void* src, size_t bytes, uint32_t* sink,
+                           hipStream_t stream);
+
+}  // namespace gufo

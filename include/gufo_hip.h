@@ -1,0 +1,213 @@
+/*
+ * gufo_hip.h - C-ABI of the MI355X (gfx950) backend for gufo-npu's quantized
+ * matrix-vector decode path.
+ *
+ * The library replaces, for this one path, what the reference engine reaches
+ * through `qwen35::Projections` (src/models/qwen35/projections.hpp:45-59): its CPU
+ * backend `GgufProjections` (src/models/qwen35/gguf_projections.cpp:179-286) and
+ * the NPU operator `npu::Q4nxGemv` (src/npu/gemv.hpp:134-158).  Weights are GGUF
+ * K-quant blocks exactly as a GGUF file stores them (row-major, Q4_K 144 B,
+ * Q5_K 176 B, Q6_K 210 B per 256 values); they are copied to HBM once and stay
+ * resident, like the NPU backend keeps its matrices on the device.
+ *
+ * Conventions
+ *   - Every entry point returns a gufo_hip_status (0 = ok) and never throws.
+ *     gufo_hip_last_error() gives the message of the calling thread's last
+ *     failure.  The C++ adapter (gufo-npu_amd/host/hip_projections.hpp) maps the
+ *     codes back to the exception types the reference throws.
+ *   - Entry points may be called from several host threads; calls are serialised
+ *     on one HIP stream, as GgufProjections serialises products on its pool
+ *     (gguf_projections.hpp:14-16).
+ *   - "_dev" variants take device pointers, enqueue on the library's stream and
+ *     return without waiting; gufo_hip_synchronize() waits.  The others take host
+ *     pointers and return when y is complete.
+ *   - x is `tokens` rows of `cols` fp32; y is `tokens` rows of fp32, a row being
+ *     the parts' outputs concatenated (projections.hpp:8-11).
+ */
+#ifndef GUFO_HIP_H_
+#define GUFO_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml tensor type ids, numerically as in GGUF (src/core/gguf.hpp:16-24). */
+enum gufo_hip_type {
+  GUFO_HIP_Q4_K = 12,
+  GUFO_HIP_Q5_K = 13,
+  GUFO_HIP_Q6_K = 14
+};
+
+/* Status codes.  The exception each one stands for in the reference:
+ *   INVALID_ARGUMENT  std::invalid_argument  partial block, unknown type
+ *                     (src/core/quant.cpp:199,224,233)
+ *   SHAPE             std::runtime_error     tensor shape mismatch
+ *                     (src/models/qwen35/gguf_projections.cpp:43)
+ *   LOGIC             std::logic_error       no weights for a stage, no such
+ *                     expert (gguf_projections.cpp:214,223,235)
+ *   NO_DEVICE         std::runtime_error     backend not available
+ *                     (src/npu/gemv_stub.cpp:8-10)
+ *   OUT_OF_RANGE      std::out_of_range      token / index out of range
+ *                     (src/models/qwen35/decoder.cpp:484)
+ */
+enum gufo_hip_status {
+  GUFO_HIP_OK = 0,
+  GUFO_HIP_ERR_NO_DEVICE = 1,
+  GUFO_HIP_ERR_NOT_INITIALIZED = 2,
+  GUFO_HIP_ERR_INVALID_ARGUMENT = 3,
+  GUFO_HIP_ERR_SHAPE = 4,
+  GUFO_HIP_ERR_LOGIC = 5,
+  GUFO_HIP_ERR_OUT_OF_RANGE = 6,
+  GUFO_HIP_ERR_OUT_OF_MEMORY = 7,
+  GUFO_HIP_ERR_RUNTIME = 8
+};
+
+/* A K-quant matrix resident in HBM.  Replaces gguf::TensorInfo + its mapped data
+ * (src/core/gguf.hpp:40-54) as GgufProjections::Rows refers to it
+ * (gguf_projections.hpp:41-45). */
+typedef struct gufo_hip_matrix gufo_hip_matrix;
+
+/* ---- life cycle ---------------------------------------------------------- */
+
+/* Selects HIP device `device`, checks that it is a gfx950 part, creates the
+ * library's stream.  Fails with NO_DEVICE where the reference's stub backend
+ * throws at construction (src/npu/gemv_stub.cpp:8-10).  Idempotent. */
+int gufo_hip_init(int device);
+/* Frees the stream and library-owned scratch.  Matrices must be destroyed first. */
+int gufo_hip_shutdown(void);
+/* Message of the calling thread's last failing call ("" if none). */
+const char* gufo_hip_last_error(void);
+/* Device name ("gfx950...") and compute-unit count of the initialised device. */
+int gufo_hip_device_info(char* name, size_t name_bytes, int* compute_units);
+
+/* ---- block geometry: quant::BlockBytes / RowBytes (src/core/quant.cpp:202-227) */
+
+/* Bytes per 256-value super-block; 0 for a type this backend does not take. */
+size_t gufo_hip_block_bytes(int ggml_type);
+/* Bytes of a row of `cols` values; 0 when cols is not a whole number of blocks
+ * (where RowBytes throws std::invalid_argument). */
+size_t gufo_hip_row_bytes(int ggml_type, size_t cols);
+
+/* ---- device memory for callers that keep x / y resident ------------------- */
+/* The NPU backend's npu::Buffer (src/npu/gemv.hpp:82-131) in four calls. */
+
+int gufo_hip_malloc(void** device_ptr, size_t bytes);
+int gufo_hip_free(void* device_ptr);
+int gufo_hip_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);
+int gufo_hip_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes);
+/* Waits for everything enqueued on the library's stream. */
+int gufo_hip_synchronize(void);
+
+/* ---- matrices ------------------------------------------------------------- */
+
+/* Copies `rows` rows of `cols` values of GGUF blocks (row-major, as stored in the
+ * file: row r starts at r * row_bytes, gguf_projections.cpp:262,269) to HBM.
+ * A 3-D expert tensor [cols, rows_per_expert, experts] is passed with
+ * rows = rows_per_expert * experts; expert e is the row range
+ * [e*rows_per_expert, (e+1)*rows_per_expert) (gguf_projections.cpp:230-233).
+ * The host bytes may be freed on return. */
+int gufo_hip_matrix_create(int ggml_type, const void* host_blocks, size_t rows,
+                           size_t cols, gufo_hip_matrix** out);
+int gufo_hip_matrix_destroy(gufo_hip_matrix* m);
+int gufo_hip_matrix_info(const gufo_hip_matrix* m, int* ggml_type, size_t* rows,
+                         size_t* cols, size_t* bytes);
+
+/* ---- the matrix-vector products ------------------------------------------- */
+
+/* GgufProjections::MatMul (gguf_projections.cpp:239-286):
+ *   y[t*stride + offset_p + r] = row (first_row[p] + r) of parts[p] . x[t]
+ * for r < n_rows[p], t < tokens, with stride = sum of n_rows and offset_p the rows
+ * of the parts before p.  All parts share `cols`.  Any tokens >= 0 is accepted;
+ * the GEMV kernels carry up to four token columns per pass over the weights.
+ * Column t of a multi-token call is bit-identical to a one-token call on x[t]. */
+int gufo_hip_gemv(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                  const size_t* n_rows, int n_parts, const float* x_host,
+                  int tokens, float* y_host);
+int gufo_hip_gemv_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                      const size_t* n_rows, int n_parts, const float* x_dev,
+                      int tokens, float* y_dev);
+
+/* Greedy pick over logits, std::max_element's rule: the first maximum wins
+ * (src/core/sampling.cpp:327-329).  `index` receives the position. */
+int gufo_hip_argmax_dev(const float* logits_dev, size_t n, int64_t* index_host);
+
+/* ---- mixture of experts ---------------------------------------------------- */
+
+/* qwen35::Route (src/models/qwen35/moe.cpp:16-42) for `tokens` rows of `experts`
+ * logits: softmax in double, the k most probable experts in order of probability
+ * (ties to the lower index), weights renormalised with the sum floored at 2^-14.
+ * ids and weights are tokens x k. */
+int gufo_hip_route_topk(const float* logits_host, int tokens, int experts, int k,
+                        int* ids_host, float* weights_host);
+int gufo_hip_route_topk_dev(const float* logits_dev, int tokens, int experts, int k,
+                            int* ids_dev, float* weights_dev);
+
+/* The grouping of Reference::Ffn (src/models/qwen35/reference.cpp:562-565), done
+ * on the device: for ids (tokens x k) writes counts[experts], offsets[experts+1]
+ * and pairs[tokens*k] - the pair ids t*k+slot grouped by expert ascending and
+ * ascending within an expert - and the number of distinct experts. */
+int gufo_hip_moe_group(const int* ids_host, int tokens, int k, int experts,
+                       int* counts_host, int* offsets_host, int* pairs_host,
+                       int* distinct_host);
+
+/* The routed part of Reference::Ffn / Decoder::MoeFfn (reference.cpp:562-606,
+ * decoder.cpp:530-558): tokens are grouped by expert on the device, every distinct
+ * expert's gate, up and down rows are streamed once over the tokens that chose it
+ * ([gate|up] -> silu(gate)*up -> down), and
+ *   y[t] = sum over slots, in slot order, of weights[t][slot] * down_out[t][slot]
+ * accumulated in double as reference.cpp:595-606 does.
+ * gate, up: experts*ffn rows x hidden; down: experts*hidden rows x ffn. */
+int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                     const gufo_hip_matrix* down, int experts, const float* x_host,
+                     int tokens, const int* ids_host, const float* weights_host,
+                     int k, float* y_host);
+int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                         const gufo_hip_matrix* down, int experts,
+                         const float* x_dev, int tokens, const int* ids_dev,
+                         const float* weights_dev, int k, float* y_dev);
+
+/* ---- prefill --------------------------------------------------------------- */
+
+/* MatMul with many tokens, the prefill shape (gguf_projections.cpp:239-286 with
+ * tokens = m; NPU analogue src/npu/gemm.hpp:99-105):
+ *   c[t*rows + r] = row r of w . a[t],  a given as bf16 (m x cols, row-major),
+ * computed on the matrix cores with fp32 accumulation.  w must be Q4_K. */
+int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host,
+                           size_t m, float* c_host);
+int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
+                               size_t m, float* c_dev);
+
+/* ---- replaying a fixed sequence of products -------------------------------- */
+
+/* A recorded sequence of "_dev" calls: the counterpart of the NPU backend's
+ * npu::Chain, which submits a layer's products as one runlist
+ * (src/npu/gemv.hpp:299-331).  Between capture_begin and capture_end the "_dev"
+ * product calls made by this thread are recorded (HIP stream capture) instead of
+ * run; graph_launch then enqueues the whole sequence with one submission.  Only the
+ * "_dev" product entry points may be called while recording, and every scratch
+ * size they need must have been seen by an earlier ordinary call (recording cannot
+ * allocate).  The buffers named at record time are the ones every replay uses. */
+typedef struct gufo_hip_graph gufo_hip_graph;
+int gufo_hip_capture_begin(void);
+int gufo_hip_capture_end(gufo_hip_graph** out);
+int gufo_hip_graph_launch(gufo_hip_graph* graph);
+int gufo_hip_graph_destroy(gufo_hip_graph* graph);
+
+/* ---- measurement ----------------------------------------------------------- */
+
+/* HIP events on the library's stream: begin records the start event, end records
+ * the stop event, waits for it and returns the milliseconds between them. */
+int gufo_hip_timer_begin(void);
+int gufo_hip_timer_end(float* milliseconds);
+/* A plain streaming read of `bytes` of device memory (sum of dwords written to
+ * *sink_dev): the achievable-read-bandwidth probe, as the reference measures its
+ * own ceiling (src/npu/device.hpp:58-74). */
+int gufo_hip_read_probe_dev(const void* src_dev, size_t bytes, uint32_t* sink_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GUFO_HIP_H_ */

@@ -1,0 +1,231 @@
+"""ctypes access to the CPU checker: the C restatement (libkquant_oracle.so) and,
+where it was built, the compiled reference (_ref/libgufo_ref.so).
+
+TEST INFRASTRUCTURE.  Only tests, the smoke check and the bench's cpu_baseline leg
+import this module; the shipped library and its Python binding never do.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent
+ORACLE_LIB = ORACLE_DIR / "libkquant_oracle.so"
+REF_LIB = ORACLE_DIR / "_ref" / "libgufo_ref.so"
+
+Q4_K, Q5_K, Q6_K = 12, 13, 14
+_SZ = C.c_size_t
+_P = C.c_void_p
+
+
+def build(ref: bool = True) -> None:
+    """make the checker libraries (the reference build is skipped where its sources
+    are absent)."""
+    targets = ["all"] + (["ref"] if ref else [])
+    subprocess.run(["make", "-s", "-C", str(ORACLE_DIR), *targets], check=True)
+
+
+_oracle = None
+_ref = None
+
+
+def lib() -> C.CDLL:
+    global _oracle
+    if _oracle is None:
+        if not ORACLE_LIB.exists():
+            build(ref=False)
+        o = C.CDLL(str(ORACLE_LIB))
+        o.gufo_oracle_half_to_float.restype = C.c_float
+        o.gufo_oracle_half_to_float.argtypes = [C.c_uint16]
+        o.gufo_oracle_block_bytes.restype = _SZ
+        o.gufo_oracle_block_bytes.argtypes = [C.c_int]
+        o.gufo_oracle_row_bytes.restype = _SZ
+        o.gufo_oracle_row_bytes.argtypes = [C.c_int, _SZ]
+        o.gufo_oracle_scale_min_k4.restype = None
+        o.gufo_oracle_scale_min_k4.argtypes = [_SZ, _P, _P, _P]
+        o.gufo_oracle_dequantize.restype = C.c_int
+        o.gufo_oracle_dequantize.argtypes = [C.c_int, _P, _P, _SZ]
+        for name in ("q4_k", "q5_k", "q6_k"):
+            fn = getattr(o, f"gufo_oracle_dot_{name}")
+            fn.restype = C.c_float
+            fn.argtypes = [_P, _P, _SZ]
+        o.gufo_oracle_dot_double.restype = C.c_double
+        o.gufo_oracle_dot_double.argtypes = [C.c_int, _P, _P, _SZ]
+        o.gufo_oracle_matmul.restype = C.c_int
+        o.gufo_oracle_matmul.argtypes = [C.c_int, _P, _P, _P, _P, _SZ, _P, C.c_int, _P,
+                                         C.c_int, C.c_int]
+        o.gufo_oracle_route.restype = None
+        o.gufo_oracle_route.argtypes = [_P, C.c_int, C.c_int, _P, _P]
+        o.gufo_oracle_argmax.restype = C.c_int64
+        o.gufo_oracle_argmax.argtypes = [_P, _SZ]
+        o.gufo_oracle_moe_group.restype = C.c_int
+        o.gufo_oracle_moe_group.argtypes = [_P, C.c_int, C.c_int, C.c_int, _P, _P, _P]
+        o.gufo_oracle_moe_ffn.restype = C.c_int
+        o.gufo_oracle_moe_ffn.argtypes = [_P, C.c_int, _P, C.c_int, _P, C.c_int, C.c_int,
+                                          C.c_int, C.c_int, _P, _P, C.c_int, C.c_int, _P, _P,
+                                          _P, C.c_int, C.c_int]
+        o.gufo_oracle_silu.restype = C.c_float
+        o.gufo_oracle_silu.argtypes = [C.c_float]
+        _oracle = o
+    return _oracle
+
+
+def ref_available() -> bool:
+    return REF_LIB.exists()
+
+
+def ref() -> C.CDLL:
+    """The compiled reference; raises FileNotFoundError where it was not built."""
+    global _ref
+    if _ref is None:
+        if not REF_LIB.exists():
+            raise FileNotFoundError(f"{REF_LIB} was not built (reference sources absent)")
+        r = C.CDLL(str(REF_LIB))
+        r.ref_half_to_float.restype = C.c_float
+        r.ref_half_to_float.argtypes = [C.c_uint16]
+        r.ref_dequantize.restype = C.c_int
+        r.ref_dequantize.argtypes = [C.c_int, _P, _P, _SZ]
+        r.ref_dot.restype = C.c_float
+        r.ref_dot.argtypes = [C.c_int, _P, _P, _SZ]
+        r.ref_route.restype = None
+        r.ref_route.argtypes = [_P, C.c_int, C.c_int, _P, _P]
+        r.ref_silu.restype = C.c_float
+        r.ref_silu.argtypes = [C.c_float]
+        r.ref_shared_expert_scale.restype = C.c_float
+        r.ref_shared_expert_scale.argtypes = [C.c_float]
+        r.ref_default_threads.restype = C.c_int
+        r.ref_usable_cpus.restype = C.c_int
+        r.ref_matmul.restype = C.c_int
+        r.ref_matmul.argtypes = [C.c_int, _P, _P, _P, _P, _SZ, _P, C.c_int, _P, C.c_int]
+        _ref = r
+    return _ref
+
+
+def _p(a: np.ndarray) -> C.c_void_p:
+    return C.c_void_p(a.ctypes.data)
+
+
+def _u8(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def half_to_float(bits: int) -> float:
+    return lib().gufo_oracle_half_to_float(bits)
+
+
+def scale_min_k4(j: int, packed: np.ndarray) -> tuple[int, int]:
+    packed = _u8(packed)
+    sc = np.zeros(1, np.uint8)
+    m = np.zeros(1, np.uint8)
+    lib().gufo_oracle_scale_min_k4(j, _p(packed), _p(sc), _p(m))
+    return int(sc[0]), int(m[0])
+
+
+def dequantize(ggml_type: int, blocks: np.ndarray, n: int, use_ref: bool = False) -> np.ndarray:
+    blocks = _u8(blocks)
+    out = np.empty(n, dtype=np.float32)
+    fn = ref().ref_dequantize if use_ref else lib().gufo_oracle_dequantize
+    if fn(ggml_type, _p(blocks), _p(out), n) != 0:
+        raise ValueError("dequantize: unknown type or partial block")
+    return out
+
+
+def dot(ggml_type: int, row: np.ndarray, x: np.ndarray, use_ref: bool = False) -> float:
+    row, x = _u8(row), _f32(x)
+    if use_ref:
+        return ref().ref_dot(ggml_type, _p(row), _p(x), x.size)
+    name = {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}[ggml_type]
+    return getattr(lib(), f"gufo_oracle_dot_{name}")(_p(row), _p(x), x.size)
+
+
+def dot_double(ggml_type: int, row: np.ndarray, x: np.ndarray) -> float:
+    row, x = _u8(row), _f32(x)
+    return lib().gufo_oracle_dot_double(ggml_type, _p(row), _p(x), x.size)
+
+
+def matmul(parts, x: np.ndarray, precision: str = "float", threads: int = 1,
+           use_ref: bool = False) -> np.ndarray:
+    """parts: sequence of (ggml_type, blocks[rows_total, row_bytes], first_row, n_rows).
+    Returns y[tokens, sum(n_rows)].  precision "float" = fused fp32 dots, "double" =
+    dequantize + double sum."""
+    x = _f32(x)
+    tokens, cols = x.shape
+    n = len(parts)
+    keep = [_u8(p[1]) for p in parts]
+    data = (C.c_void_p * n)(*[k.ctypes.data for k in keep])
+    types = (C.c_int * n)(*[int(p[0]) for p in parts])
+    first = (C.c_size_t * n)(*[int(p[2]) for p in parts])
+    rows = (C.c_size_t * n)(*[int(p[3]) for p in parts])
+    y = np.empty((tokens, sum(int(p[3]) for p in parts)), dtype=np.float32)
+    if use_ref:
+        if precision != "float":
+            raise ValueError("the reference driver runs the fused fp32 dots only")
+        status = ref().ref_matmul(n, data, types, first, rows, cols, _p(x), tokens, _p(y),
+                                  threads)
+    else:
+        status = lib().gufo_oracle_matmul(n, data, types, first, rows, cols, _p(x), tokens,
+                                          _p(y), 1 if precision == "double" else 0, threads)
+    if status != 0:
+        raise ValueError("matmul: bad argument")
+    return y
+
+
+def route(logits: np.ndarray, k: int, use_ref: bool = False):
+    logits = _f32(logits)
+    tokens, experts = logits.shape
+    ids = np.empty((tokens, k), dtype=np.int32)
+    weights = np.empty((tokens, k), dtype=np.float32)
+    fn = ref().ref_route if use_ref else lib().gufo_oracle_route
+    for t in range(tokens):
+        fn(_p(logits[t]), experts, k, _p(ids[t]), _p(weights[t]))
+    return ids, weights
+
+
+def argmax(v: np.ndarray) -> int:
+    v = _f32(v)
+    return lib().gufo_oracle_argmax(_p(v), v.size)
+
+
+def moe_group(ids: np.ndarray, experts: int):
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    tokens, k = ids.shape
+    counts = np.empty(experts, np.int32)
+    offsets = np.empty(experts + 1, np.int32)
+    pairs = np.empty(tokens * k, np.int32)
+    distinct = lib().gufo_oracle_moe_group(_p(ids), tokens, k, experts, _p(counts),
+                                           _p(offsets), _p(pairs))
+    return counts, offsets, pairs, distinct
+
+
+def moe_ffn(gate, gate_type, up, up_type, down, down_type, experts, hidden, ffn, logits, x,
+            k, precision: str = "float", threads: int = 1):
+    gate, up, down = _u8(gate), _u8(up), _u8(down)
+    logits, x = _f32(logits), _f32(x)
+    tokens = x.shape[0]
+    ids = np.empty((tokens, k), np.int32)
+    weights = np.empty((tokens, k), np.float32)
+    y = np.empty((tokens, hidden), np.float32)
+    status = lib().gufo_oracle_moe_ffn(_p(gate), gate_type, _p(up), up_type, _p(down),
+                                       down_type, experts, hidden, ffn, _p(logits), _p(x),
+                                       tokens, k, _p(ids), _p(weights), _p(y),
+                                       1 if precision == "double" else 0, threads)
+    if status != 0:
+        raise ValueError("moe_ffn: bad argument")
+    return ids, weights, y
+
+
+def silu(x: float) -> float:
+    return lib().gufo_oracle_silu(x)
+
+
+def rel_l2(got: np.ndarray, want: np.ndarray) -> float:
+    got = np.asarray(got, dtype=np.float64).ravel()
+    want = np.asarray(want, dtype=np.float64).ravel()
+    return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-300))

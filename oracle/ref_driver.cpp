@@ -1,0 +1,156 @@
+// TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+//
+// C entry points over the reference's own implementation of the quantized
+// matrix-vector path, compiled from the reference's sources where they lie
+// (see Makefile: -I$(REFERENCE)/src plus its core/quant.cpp and
+// models/qwen35/moe.cpp).  Nothing of the reference is copied here: this file
+// only calls it.  The result, oracle/_ref/libgufo_ref.so, validates the C
+// restatement in kquant_oracle.c and is the "reference" CPU baseline the bench
+// times beside the GPU.
+//
+// What is the reference's and what is this driver's:
+//   * ref_half_to_float, ref_dequantize, ref_dot, ref_route, ref_silu and
+//     ref_shared_expert_scale call quant::HalfToFloat, quant::Dequantize,
+//     gguf_dot::DotQ4_K/DotQ5_K/DotQ6_K (the AVX2+FMA+F16C bodies, built with
+//     -march=x86-64-v3 as the reference builds them), qwen35::Route, simd::Silu
+//     and qwen35::SharedExpertScale.
+//   * ref_matmul runs those dots over row ranges on the reference's SpinPool
+//     (core/thread_pool.hpp) in jobs of 16 rows and writes
+//     y[t*stride + offset + r], the loop of GgufProjections::MatMul
+//     (models/qwen35/gguf_projections.cpp:239-286); the loop itself is restated
+//     here because MatMul is a private member that needs a whole model file.
+#include <algorithm>
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <vector>
+
+#include "core/cpus.hpp"
+#include "core/quant.hpp"
+#include "core/simd.hpp"
+#include "core/thread_pool.hpp"
+#include "models/qwen35/gguf_dot.hpp"
+#include "models/qwen35/moe.hpp"
+
+namespace {
+
+using gufo_npu::gguf::GgmlType;
+namespace dot = gufo_npu::qwen35::gguf_dot;
+
+using RowDot = float (*)(const std::uint8_t*, const float*, std::size_t);
+
+RowDot DotFor(int type) {
+  switch (static_cast<GgmlType>(type)) {
+    case GgmlType::kQ4_K: return &dot::DotQ4_K;
+    case GgmlType::kQ5_K: return &dot::DotQ5_K;
+    case GgmlType::kQ6_K: return &dot::DotQ6_K;
+    default: return nullptr;
+  }
+}
+
+struct Pool {
+  explicit Pool(std::size_t workers) : pool(workers) {}
+  gufo_npu::SpinPool pool;
+  std::mutex run;
+};
+
+std::mutex g_pools_mutex;
+std::vector<std::unique_ptr<Pool>> g_pools;  // index = threads
+
+// A pool of `threads` threads in all (the caller included), kept for reuse.
+Pool& PoolFor(std::size_t threads) {
+  const std::lock_guard<std::mutex> lock(g_pools_mutex);
+  if (g_pools.size() <= threads) g_pools.resize(threads + 1);
+  if (!g_pools[threads]) g_pools[threads] = std::make_unique<Pool>(threads - 1);
+  return *g_pools[threads];
+}
+
+}  // namespace
+
+extern "C" {
+
+float ref_half_to_float(std::uint16_t h) { return gufo_npu::quant::HalfToFloat(h); }
+
+int ref_dequantize(int type, const std::uint8_t* src, float* dst, std::size_t n) {
+  try {
+    gufo_npu::quant::Dequantize(static_cast<GgmlType>(type), src, dst, n);
+    return 0;
+  } catch (...) {
+    return -1;
+  }
+}
+
+float ref_dot(int type, const std::uint8_t* row, const float* x, std::size_t n) {
+  const RowDot fn = DotFor(type);
+  return fn != nullptr ? fn(row, x, n) : 0.0f;
+}
+
+void ref_route(const float* logits, int experts, int k, int* chosen,
+               float* weights) {
+  gufo_npu::qwen35::Route(logits, experts, k, chosen, weights);
+}
+
+// core/simd.hpp:82-84: x / (1 + e^-x) in fp32.
+float ref_silu(float x) { return gufo_npu::simd::Silu(x); }
+
+float ref_shared_expert_scale(float logit) {
+  return gufo_npu::qwen35::SharedExpertScale(logit);
+}
+
+// The reference's thread policy for these products: the caller plus
+// HalfCpuWorkers() (core/cpus.hpp:53-55, gguf_projections.cpp:93-98).
+int ref_default_threads() {
+  return static_cast<int>(gufo_npu::HalfCpuWorkers() + 1);
+}
+
+int ref_usable_cpus() { return static_cast<int>(gufo_npu::UsableCpus()); }
+
+// threads <= 0 selects ref_default_threads().
+int ref_matmul(int n_parts, const std::uint8_t* const* data, const int* types,
+               const std::size_t* first, const std::size_t* rows, std::size_t in,
+               const float* x, int tokens, float* y, int threads) {
+  constexpr std::size_t kChunk = 16;
+  if (n_parts <= 0 || tokens < 0) return -1;
+  std::vector<std::size_t> first_job = {0};
+  std::size_t stride = 0;
+  for (int p = 0; p < n_parts; ++p) {
+    if (DotFor(types[p]) == nullptr) return -1;
+    stride += rows[p];
+    first_job.push_back(first_job.back() + (rows[p] + kChunk - 1) / kChunk);
+  }
+  std::size_t row_bytes_of[64];
+  if (n_parts > 64) return -1;
+  try {
+    for (int p = 0; p < n_parts; ++p) {
+      row_bytes_of[p] =
+          gufo_npu::quant::RowBytes(static_cast<GgmlType>(types[p]), in);
+    }
+  } catch (...) {
+    return -1;
+  }
+  Pool& pool = PoolFor(threads > 0 ? static_cast<std::size_t>(threads)
+                                   : static_cast<std::size_t>(ref_default_threads()));
+  const std::lock_guard<std::mutex> lock(pool.run);
+  pool.pool.Run(first_job.back(), [&](std::size_t job) {
+    std::size_t p = 0;
+    std::size_t offset = 0;
+    while (job >= first_job[p + 1]) {
+      offset += rows[p];
+      ++p;
+    }
+    const RowDot fused = DotFor(types[p]);
+    const std::size_t begin = (job - first_job[p]) * kChunk;
+    const std::size_t end = std::min(rows[p], begin + kChunk);
+    for (std::size_t r = begin; r < end; ++r) {
+      const std::uint8_t* row = data[p] + (first[p] + r) * row_bytes_of[p];
+      for (int t = 0; t < tokens; ++t) {
+        y[static_cast<std::size_t>(t) * stride + offset + r] =
+            fused(row, x + static_cast<std::size_t>(t) * in, in);
+      }
+    }
+  });
+  return 0;
+}
+
+}  // extern "C"
