@@ -258,7 +258,7 @@ def gemv(parts: Sequence[Part], x: np.ndarray, tokens: int | None = None) -> np.
     if tokens is None:
         tokens = x.shape[0] if x.ndim == 2 else 1
     stride = sum(int(p[2]) for p in parts)
-    y = np.empty((tokens, stride), dtype=np.float32)
+    y = np.empty((max(tokens, 0), stride), dtype=np.float32)
     handles, first, rows, n = _parts_arrays(parts)
     _check(load_library().gufo_hip_gemv(handles, first, rows, n, _ptr(x), tokens, _ptr(y)))
     return y

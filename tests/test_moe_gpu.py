@@ -18,6 +18,18 @@ def say(*args):
     print(*args, flush=True)
 
 
+def same(a, b) -> bool:
+    """Exact equality as a bool, so a failure prints no arrays."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    if a.dtype == np.float32:
+        a, b = a.view(np.uint32), b.view(np.uint32)
+    return bool(np.array_equal(a, b))
+
+
+def close(a, b, rtol=1e-6) -> bool:
+    return bool(np.allclose(a, b, rtol=rtol, atol=0))
+
+
 def engineered_logits():
     # The rows tests/golden/make_golden.py routes through the reference.
     logits = synth.router_logits(64, cfg.EXPERTS4, cfg.SEED + 180)
@@ -35,11 +47,11 @@ def test_route_indices_bit_exact_against_reference_golden(hip, oracle):
     golden = np.load(GOLDEN / "config4_moe.npz")
     logits = engineered_logits()
     ids, weights = hip.route_topk(logits, cfg.TOPK4)
-    assert np.array_equal(ids, golden["route_ids"])
-    assert np.allclose(weights, golden["route_weights"], rtol=1e-6, atol=0)
+    assert same(ids, golden["route_ids"])
+    assert close(weights, golden["route_weights"])
     want_ids, want_w = oracle.route(logits, cfg.TOPK4)
-    assert np.array_equal(ids, want_ids)
-    assert np.allclose(weights, want_w, rtol=1e-6, atol=0)
+    assert same(ids, want_ids)
+    assert close(weights, want_w)
 
 
 @pytest.mark.parametrize("experts,k", [(8, 1), (8, 8), (60, 6), (64, 8), (256, 8), (1000, 17)])
@@ -51,9 +63,9 @@ def test_route_shapes_and_ties(hip, oracle, experts, k):
     logits[2] = np.round(logits[2] * 2) / 2           # many duplicate values
     ids, weights = hip.route_topk(logits, k)
     want_ids, want_w = oracle.route(logits, k)
-    assert np.array_equal(ids, want_ids)
+    assert same(ids, want_ids)
     assert list(ids[0]) == list(range(k))
-    assert np.allclose(weights, want_w, rtol=1e-6, atol=0)
+    assert close(weights, want_w)
     assert np.allclose(weights.sum(axis=1), 1.0, atol=1e-5)
 
 
@@ -64,16 +76,16 @@ def test_group_tables_exact(hip, oracle):
         ids = np.stack([gen.permutation(experts)[:k] for _ in range(tokens)]).astype(np.int32)
         counts, offsets, pairs, distinct = hip.moe_group(ids, experts)
         w_counts, w_offsets, w_pairs, w_distinct = oracle.moe_group(ids, experts)
-        assert np.array_equal(counts, w_counts)
-        assert np.array_equal(offsets, w_offsets)
-        assert np.array_equal(pairs, w_pairs)
+        assert same(counts, w_counts)
+        assert same(offsets, w_offsets)
+        assert same(pairs, w_pairs)
         assert distinct == w_distinct
     golden = np.load(GOLDEN / "config4_moe.npz")
     for b in (1, 4):
         counts, offsets, pairs, distinct = hip.moe_group(golden[f"ids_b{b}"], cfg.EXPERTS4)
-        assert np.array_equal(counts, golden[f"counts_b{b}"])
-        assert np.array_equal(offsets, golden[f"offsets_b{b}"])
-        assert np.array_equal(pairs, golden[f"pairs_b{b}"])
+        assert same(counts, golden[f"counts_b{b}"])
+        assert same(offsets, golden[f"offsets_b{b}"])
+        assert same(pairs, golden[f"pairs_b{b}"])
         assert distinct == int(golden[f"distinct_b{b}"])
 
 
@@ -102,16 +114,15 @@ def test_moe_ffn_small_with_crowded_experts(hip, oracle):
     want_ids, want_w, want_y = oracle.moe_ffn(gate, synth.Q4_K, up, synth.Q4_K, down,
                                               synth.Q5_K, experts, hidden, ffn, logits, x, k,
                                               precision="double")
-    assert np.array_equal(ids, want_ids)
+    assert same(ids, want_ids)
     assert int(np.max(np.bincount(ids.reshape(-1), minlength=experts))) > 4
     y = hip.moe_ffn(mg, mu, md, experts, x, ids, weights)
     assert oracle.rel_l2(y, want_y) <= TOLERANCE
     # grouped batch == per-token calls, bit for bit; repeats too
     for t in range(tokens):
         single = hip.moe_ffn(mg, mu, md, experts, x[t:t + 1], ids[t:t + 1], weights[t:t + 1])
-        assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32))
-    assert np.array_equal(y.view(np.uint32),
-                          hip.moe_ffn(mg, mu, md, experts, x, ids, weights).view(np.uint32))
+        assert same(single[0], y[t])
+    assert same(y, hip.moe_ffn(mg, mu, md, experts, x, ids, weights))
     with pytest.raises(hip.LogicError):
         bad = ids.copy()
         bad[0, 0] = experts
@@ -137,8 +148,8 @@ def test_config4_moe_expert_gemv(hip, oracle):
         x = synth.activations(tokens, cfg.HIDDEN4, cfg.CONFIG4_X_SEED + tokens)
         x = x * np.float32(cfg.CONFIG4_X_SCALE)
         ids, weights = hip.route_topk(logits, cfg.TOPK4)
-        assert np.array_equal(ids, golden[f"ids_b{tokens}"])
-        assert np.allclose(weights, golden[f"weights_b{tokens}"], rtol=1e-6, atol=0)
+        assert same(ids, golden[f"ids_b{tokens}"])
+        assert close(weights, golden[f"weights_b{tokens}"])
         y = hip.moe_ffn(mg, mu, md, cfg.EXPERTS4, x, ids, weights)
         assert oracle.rel_l2(y, golden[f"y_b{tokens}"]) <= TOLERANCE
         _, _, want = oracle.moe_ffn(wg, gate.ggml_type, wu, up.ggml_type, wd, down.ggml_type,
@@ -148,6 +159,6 @@ def test_config4_moe_expert_gemv(hip, oracle):
         for t in range(tokens):
             single = hip.moe_ffn(mg, mu, md, cfg.EXPERTS4, x[t:t + 1], ids[t:t + 1],
                                  weights[t:t + 1])
-            assert np.array_equal(single[0].view(np.uint32), y[t].view(np.uint32))
+            assert same(single[0], y[t])
     for m in (mg, mu, md):
         m.destroy()
