@@ -85,8 +85,9 @@ __global__ __launch_bounds__(256) void ReadProbe(const U32x4* __restrict__ src,
     const U32x4 a = src[i];
     acc ^= a.x ^ a.y ^ a.z ^ a.w;
   }
-  for (int off = 32; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, 64);
-  if ((threadIdx.x & 63) == 0) atomicXor(sink, acc);
+  // The loads must stay alive, the store must (almost) never happen: an atomic per
+  // wave on one address would time the atomics, not the reads.
+  if (acc == 0x9E3779B9u) *sink = acc;
 }
 
 }  // namespace

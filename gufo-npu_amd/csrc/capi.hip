@@ -215,8 +215,20 @@ int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
   }
   const size_t cols = parts[0]->cols;
-  for (int t0 = 0; t0 < tokens; t0 += kMaxGemvTokens) {
-    const int nt = tokens - t0 < kMaxGemvTokens ? tokens - t0 : kMaxGemvTokens;
+  // Token columns per pass over the weights: what the narrowest type's LDS need
+  // allows for rows this wide.
+  int per_pass = kMaxGemvTokens;
+  for (int p = 0; p < n_parts; ++p) {
+    const int fit = gufo::GemvMaxTokens(parts[p]->type,
+                                        static_cast<uint32_t>(cols / gufo::kSuperBlock));
+    if (fit < per_pass) per_pass = fit;
+  }
+  if (per_pass < 1) {
+    return Fail(GUFO_HIP_ERR_SHAPE, "rows of %zu values exceed what one workgroup can stage",
+                cols);
+  }
+  for (int t0 = 0; t0 < tokens; t0 += per_pass) {
+    const int nt = tokens - t0 < per_pass ? tokens - t0 : per_pass;
     size_t offset = 0;
     int p = 0;
     while (p < n_parts) {

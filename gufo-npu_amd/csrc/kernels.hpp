@@ -25,8 +25,16 @@ struct GemvLaunch {
   uint32_t y_stride;        // floats between token rows of y
 };
 
+// LDS a product kernel may use: the whole LDS of a gfx950 compute unit.
+constexpr size_t kGemvMaxLdsBytes = 160 * 1024;
+
+// Token columns one launch can carry for rows of blocks_per_row super-blocks: the
+// quantized activation rows of all columns must fit in LDS together (at most
+// kMaxGemvTokens).
+int GemvMaxTokens(int type, uint32_t blocks_per_row);
+
 // y[t*y_stride + part.y_offset + r] = row r of part . x[t*cols ...], t < tokens.
-// All parts are of `type`.  tokens in 1..kMaxGemvTokens.
+// All parts are of `type`.  tokens in 1..GemvMaxTokens(type, blocks_per_row).
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream);
 
@@ -92,7 +100,8 @@ constexpr int kArgmaxBlocks = 1024;
 hipError_t LaunchArgmax(const float* v, size_t n, void* scratch, int64_t* out,
                         hipStream_t stream);
 
-// Streaming read of `bytes` (multiple of 16) -> xor of all dwords into *sink.
+// Streaming read of `bytes` (multiple of 16); *sink is written only if a lane's
+// xor of its dwords equals a magic constant, which keeps the loads alive.
 hipError_t LaunchReadProbe(const void* src, size_t bytes, uint32_t* sink,
                            hipStream_t stream);
 

@@ -6,23 +6,37 @@
 // y[t*stride + offset + r] = row r . x[t].  Q4_K / Q5_K / Q6_K super-blocks are
 // unpacked in registers; nothing is dequantized to memory.
 //
-// Work decomposition (wave64):
-//   * A super-block (256 weights) is decoded by 8 consecutive lanes, 32 weights
-//     each, so that every lane's share of the quant bytes is one or three
-//     contiguous vector loads and consecutive lanes read consecutive addresses.
-//   * A wave pass covers 8 super-blocks: `bpp` consecutive blocks of each of
-//     8/bpp consecutive rows, bpp = the largest power of two <= 8 dividing
-//     cols/256.  For cols = 2048 one pass is exactly one row; for the 512-wide
-//     expert down projection it is four rows.
-//   * The activation rows (all token columns) are staged in LDS once per
-//     workgroup and K-chunk together with the sums of every 8 consecutive values,
-//     which carry the Q4_K/Q5_K minimum term and Q6_K's -32 code offset.
-//   * Each weight register is decoded once and applied to every token column.
-//   * Per-row totals are reduced with wavefront shuffles in a fixed order.
+// The kernel is bound by the HBM read of the packed weights, so everything else is
+// arranged to keep that stream saturated:
 //
-// The arithmetic per token column does not depend on how many columns travel
+//   * Persistent waves.  A launch has at most a few workgroups per compute unit;
+//     every wave walks the rows in a grid-stride loop and keeps kDepth row visits
+//     of weight loads in flight in registers (issue the loads of visit i+kDepth,
+//     then do the arithmetic of visit i).
+//   * Four lanes per super-block, 64 weights per lane, 16 super-blocks per wave
+//     pass.  Each lane's share of a block is two or three 16-byte loads (Q6_K
+//     blocks are 210 bytes, so those loads are only 2-byte aligned, which gfx950
+//     global loads accept).  A pass covers `bpp` consecutive blocks of each of
+//     16/bpp consecutive rows, bpp = the largest power of two <= 16 dividing
+//     cols/256: one pass is two whole rows for cols = 2048 and eight rows for the
+//     512-wide expert down projection.
+//   * Integer dot products.  The activation row is quantized once per workgroup
+//     into three signed 8-bit limbs per value (a 21-bit integer X with a power-of-
+//     two scale per scale group of the weight format: 32 values for Q4_K/Q5_K, 16
+//     for Q6_K), staged in LDS in the order the lanes read it, and then held in
+//     registers.  The 4/5/6-bit codes are already bytes after unpacking, so a
+//     sub-block's sum(code * X) is exact integer arithmetic on v_dot4_i32_i8, 0.75
+//     instructions per weight and token instead of a convert and an fma each.  The
+//     sub-block sums are converted to fp32 once, scaled (d*sc, the x scale) and
+//     accumulated in fp32 across sub-blocks, super-blocks and lanes.  Unit-vector
+//     inputs reproduce the dequantized weights bit for bit; for N(0,1) inputs the
+//     result is within ~5e-7 (rel-L2) of the double-precision product.
+//   * Each decoded weight register is applied to every token column (up to four).
+//   * Per-row totals are reduced across lanes with DPP adds in a fixed order.
+//
+// The arithmetic of a token column does not depend on how many columns travel
 // together, so column t of an N-column call equals the one-column call bit for
-// bit.
+// bit, and repeated calls give identical bits.
 #include "kernels.hpp"
 #include "kquant_common.hpp"
 
@@ -30,315 +44,579 @@ namespace gufo {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
-constexpr int kVisits = 4;  // row groups each wave owns within a workgroup
-constexpr int kLdsBudget = 48 * 1024;
-// LDS floats per staged super-block and token: 256 values + 32 sums of 8.
-constexpr int kLdsFloatsPerBlock = 256 + 32;
+constexpr int kWavesPerGroup = kThreads / 64;
+constexpr int kDepth = 4;          // row visits of weight loads in flight per wave
+constexpr int kBlocksPerPass = 16;  // super-blocks a wave covers per pass (4 lanes each)
+constexpr uint32_t kMaxGrid = 512;  // persistent workgroups of a dense launch
 
 struct GemvParams {
   GemvLaunch launch;
+  uint32_t start[kMaxGemvParts];  // first flat row of each part
   uint32_t row_bytes;
   uint32_t cols;
-  uint32_t bpp_log2;      // blocks of one row per wave pass = 1 << bpp_log2
-  uint32_t rows_per_wg;   // kVisits * kWaves * (8 >> bpp_log2)
-  uint32_t chunk_blocks;  // super-blocks of x staged at a time
+  uint32_t bpp_log2;  // blocks of one row per wave pass = 1 << bpp_log2 (<= 16)
+  uint32_t passes;    // blocks_per_row >> bpp_log2
+  uint32_t n_groups;  // row groups = ceil(total_rows / rows per pass)
 };
 
 __device__ __forceinline__ float Fma(float a, float b, float c) {
   return __builtin_fmaf(a, b, c);
 }
 
-// Sum of four byte codes times four activations, added to acc.
-__device__ __forceinline__ float Dot4Bytes(uint32_t codes, float4 x, float acc) {
-  acc = Fma(Byte0(codes), x.x, acc);
-  acc = Fma(Byte1(codes), x.y, acc);
-  acc = Fma(Byte2(codes), x.z, acc);
-  acc = Fma(Byte3(codes), x.w, acc);
-  return acc;
+__device__ __forceinline__ int Dot4(uint32_t codes, uint32_t limbs, int acc) {
+  return __builtin_amdgcn_sdot4(static_cast<int>(codes), static_cast<int>(limbs), acc,
+                                false);
 }
 
-// ---- Q4_K / Q5_K ------------------------------------------------------------
-// Lane `sub` (0..7) of a block takes 16 of the 128 quant bytes: run p = sub/2 of
-// 32 bytes (sub-blocks 2p from the low nibbles and 2p+1 from the high nibbles),
-// half h = sub%2 of that run, i.e. values 16h..16h+15 of both sub-blocks.
-// weight = (d*sc_j)*q - (dmin*m_j), so a sub-block contributes
-// (d*sc_j) * sum(q*x) - (dmin*m_j) * sum(x).
-template <bool kFifthBit, int NTOK>
-__device__ __forceinline__ void MacK4(const uint8_t* blk, int sub, const float* xb,
-                                      const float* sb, int x_stride, int s_stride,
-                                      float (&acc)[NTOK]) {
-  const int p = sub >> 1;
-  const int h = sub & 1;
-  const U32x4 hdr = Load16(blk);
-  const U32x4 q = Load16(blk + 16 + (kFifthBit ? 32 : 0) + 32 * p + 16 * h);
-  U32x4 high = {0, 0, 0, 0};
-  if (kFifthBit) high = Load16(blk + 16 + 16 * h);
+__device__ __forceinline__ float Silu(float v) { return v / (1.0f + expf(-v)); }
 
-  const float d = HalfBitsToFloat(hdr.x & 0xFFFFu);
-  const float dmin = HalfBitsToFloat(hdr.x >> 16);
-  uint32_t sc0, m0, sc1, m1;
-  ScaleMinK4(hdr.y, hdr.z, hdr.w, 2 * p, &sc0, &m0);
-  ScaleMinK4(hdr.y, hdr.z, hdr.w, 2 * p + 1, &sc1, &m1);
-  const float scale0 = d * static_cast<float>(sc0);
-  const float scale1 = d * static_cast<float>(sc1);
-  const float min0 = dmin * static_cast<float>(m0);
-  const float min1 = dmin * static_cast<float>(m1);
+// ---- the quantized activation row ---------------------------------------------
+//
+// x = s * X with s a power of two and |X| <= 2^20, X = a0 + 256 a1 + 65536 a2 with
+// signed bytes a0, a1 in [-128, 127] and a2 in [-16, 16].  The bytes of four
+// consecutive values share a dword per limb, the operand layout of v_dot4_i32_i8.
+//
+// Per lane (64 values of one super-block):
+//   Q4_K/Q5_K  lane p owns sub-blocks 2p and 2p+1: limb[half][limb][8 dwords],
+//              xs[half] = s, fx[half] = s * sum(X) (carries the minimum term)
+//              = 52 dwords, 13 LDS slots of 16 bytes
+//   Q6_K       lane (n, i) owns the four 16-value groups 128n + 32k + 16i:
+//              limb[k][limb][4 dwords], xs[k] = s, sx32[k] = 32 * sum(X) (carries
+//              the -32 code offset) = 56 dwords, 14 slots
+// LDS holds [token][pass][slot][position] x 16 bytes, position = blk_lane*4 + lane
+// within the block, so one ds_read_b128 per slot is conflict free.
 
-  uint32_t lo[4];
-  uint32_t hi[4];
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    lo[w] = q[w] & 0x0F0F0F0Fu;
-    hi[w] = (q[w] >> 4) & 0x0F0F0F0Fu;
-    if (kFifthBit) {
-      lo[w] |= ((high[w] >> (2 * p)) & 0x01010101u) << 4;
-      hi[w] |= ((high[w] >> (2 * p + 1)) & 0x01010101u) << 4;
-    }
-  }
-#pragma unroll
-  for (int t = 0; t < NTOK; ++t) {
-    const float4* xl =
-        reinterpret_cast<const float4*>(xb + t * x_stride + 64 * p + 16 * h);
-    const float4* xh = xl + 8;  // +32 values
-    float dot_lo = 0.0f;
-    float dot_hi = 0.0f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      dot_lo = Dot4Bytes(lo[w], xl[w], dot_lo);
-      dot_hi = Dot4Bytes(hi[w], xh[w], dot_hi);
-    }
-    const float* s = sb + t * s_stride + 8 * p + 2 * h;
-    const float sum_lo = s[0] + s[1];
-    const float sum_hi = s[4] + s[5];
-    float part = scale0 * dot_lo;
-    part = Fma(-min0, sum_lo, part);
-    part = Fma(scale1, dot_hi, part);
-    part = Fma(-min1, sum_hi, part);
-    acc[t] += part;
-  }
+struct XK4 {
+  uint32_t limb[2][3][8];
+  float xs[2];
+  float fx[2];
+};
+
+struct XQ6 {
+  uint32_t limb[4][3][4];
+  float xs[4];
+  int sx32[4];
+};
+
+template <int TYPE>
+struct XOf {
+  using Type = XK4;
+};
+template <>
+struct XOf<kTypeQ6K> {
+  using Type = XQ6;
+};
+
+template <int TYPE>
+__host__ __device__ constexpr int Slots() {
+  return TYPE == kTypeQ6K ? 14 : 13;
 }
 
-// ---- Q6_K -------------------------------------------------------------------
-// Lane `sub` (0..7): half n = sub/4 of the block (128 values), eighth i = sub%4.
-// It reads ql[64n+8i..+8), ql[64n+32+8i..+8) and qh[32n+8i..+8) and so owns
-// values 128n + 32k + 8i + c for k < 4, c < 8: code = 4 low bits from the first
-// (k even) or second (k odd) ql run, low nibble for k < 2 and high nibble
-// otherwise, plus bits 2k..2k+1 of qh.  weight = d * sc[8n + 2k + i/2] * (code-32).
-template <int NTOK>
-__device__ __forceinline__ void MacQ6K(const uint8_t* blk, int sub, const float* xb,
-                                       const float* sb, int x_stride, int s_stride,
-                                       float (&acc)[NTOK]) {
-  const int n = sub >> 2;
-  const int i = sub & 3;
-  const U32x2 a = Load8Align2(blk + 64 * n + 8 * i);
-  const U32x2 b = Load8Align2(blk + 64 * n + 32 + 8 * i);
-  const U32x2 hq = Load8Align2(blk + 128 + 32 * n + 8 * i);
-  const U32x2 sc8 = Load8Align2(blk + 192 + 8 * n);
-  const float d = HalfBitsToFloat(Load2(blk + 208));
+// The power-of-two scale 2^e with gmax * 2^-e in [2^19, 2^20), and its inverse.
+// Groups whose largest magnitude is below 2^-107 quantize to zero.
+__device__ __forceinline__ void GroupScale(float gmax, float* scale, float* inverse) {
+  const uint32_t exponent = (__float_as_uint(gmax) >> 23) & 0xFFu;
+  const bool live = exponent >= 20u && exponent < 255u;
+  *scale = live ? __uint_as_float((exponent - 19u) << 23) : 0.0f;
+  *inverse = live ? __uint_as_float((273u - exponent) << 23) : 0.0f;
+}
 
-  uint32_t codes[4][2];
-  float scale[4];
+// Lane exchange inside a quad (DPP quad_perm), for the group-wide max and sum below.
+template <int kCtrl>
+__device__ __forceinline__ int QuadSwap(int v) {
+  return __builtin_amdgcn_mov_dpp(v, kCtrl, 0xF, 0xF, true);
+}
+
+// Quantizes the 8 consecutive activations of one thread, given the largest magnitude
+// of the whole scale group: two dwords per limb, the scale and the sum of the X.
+__device__ __forceinline__ void QuantizeOctet(const float (&v)[8], float gmax,
+                                              uint32_t (&limb)[3][2], float* scale,
+                                              int* sum) {
+  float s, inv;
+  GroupScale(gmax, &s, &inv);
+  int total = 0;
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
-    codes[0][w] = (a[w] & 0x0F0F0F0Fu) | ((hq[w] << 4) & 0x30303030u);
-    codes[1][w] = (b[w] & 0x0F0F0F0Fu) | ((hq[w] << 2) & 0x30303030u);
-    codes[2][w] = ((a[w] >> 4) & 0x0F0F0F0Fu) | (hq[w] & 0x30303030u);
-    codes[3][w] = ((b[w] >> 4) & 0x0F0F0F0Fu) | ((hq[w] >> 2) & 0x30303030u);
+    limb[0][w] = 0;
+    limb[1][w] = 0;
+    limb[2][w] = 0;
   }
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    // int8 scale number 2k + i/2 of this half's eight.
-    const uint32_t word = k < 2 ? sc8.x : sc8.y;
-    const int shift = 8 * (((2 * k) & 3) + (i >> 1));
-    const int sc = static_cast<int>(word << (24 - shift)) >> 24;
-    scale[k] = static_cast<float>(sc);
+  for (int c = 0; c < 8; ++c) {
+    const int x0 = __float2int_rn(v[c] * inv);
+    const int x1 = (x0 + 128) >> 8;
+    const int x2 = (x1 + 128) >> 8;
+    total += x0;
+    const int shift = 8 * (c & 3);
+    limb[0][c >> 2] |= static_cast<uint32_t>(x0 & 0xFF) << shift;
+    limb[1][c >> 2] |= static_cast<uint32_t>(x1 & 0xFF) << shift;
+    limb[2][c >> 2] |= static_cast<uint32_t>(x2 & 0xFF) << shift;
   }
-#pragma unroll
-  for (int t = 0; t < NTOK; ++t) {
-    const float* xt = xb + t * x_stride + 128 * n + 8 * i;
-    const float* st = sb + t * s_stride + 16 * n + i;
-    float block = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float4* xv = reinterpret_cast<const float4*>(xt + 32 * k);
-      float group = Dot4Bytes(codes[k][0], xv[0], 0.0f);
-      group = Dot4Bytes(codes[k][1], xv[1], group);
-      group = Fma(-32.0f, st[4 * k], group);
-      block = Fma(scale[k], group, block);
-    }
-    acc[t] = Fma(d, block, acc[t]);
-  }
-}
-
-template <int TYPE, int NTOK>
-__device__ __forceinline__ void MacBlock(const uint8_t* blk, int sub, const float* xb,
-                                         const float* sb, int x_stride, int s_stride,
-                                         float (&acc)[NTOK]) {
-  if (TYPE == kTypeQ4K) {
-    MacK4<false, NTOK>(blk, sub, xb, sb, x_stride, s_stride, acc);
-  } else if (TYPE == kTypeQ5K) {
-    MacK4<true, NTOK>(blk, sub, xb, sb, x_stride, s_stride, acc);
-  } else {
-    MacQ6K<NTOK>(blk, sub, xb, sb, x_stride, s_stride, acc);
-  }
+  *scale = s;
+  *sum = total;
 }
 
 // Where the token columns of one kernel instance live: x[t] is the activation row
-// of column t, y[t] the output row (the kernel adds part.y_offset + r).
+// of column t, y[t] the output row.
 template <int NTOK>
 struct Columns {
   const float* x[NTOK];
   float* y[NTOK];
 };
 
-__device__ __forceinline__ float Silu(float v) { return v / (1.0f + expf(-v)); }
+template <int NTOK>
+__device__ __forceinline__ const float* ColumnX(const Columns<NTOK>& col, uint32_t t) {
+  const float* p = col.x[0];
+#pragma unroll
+  for (int i = 1; i < NTOK; ++i) {
+    if (t == static_cast<uint32_t>(i)) p = col.x[i];
+  }
+  return p;
+}
 
-// One workgroup's share of the product.  kSwiGlu: x[t] points at a [gate | up] row
-// of 2*cols values and the activation staged in LDS is silu(gate) * up, the step
-// between an expert's two products (src/models/qwen35/decoder.cpp:547-549 of the
-// reference).  part_shift is added to every part's row pointer (the byte offset
-// of an expert's rows inside a 3-D tensor).
+// Loads kValues activations; with kSwiGlu the row holds [gate | up] (2*cols values)
+// and the activation is silu(gate) * up, the step between an expert's two products
+// (src/models/qwen35/decoder.cpp:547-549 of the reference).
+template <int kValues, bool kSwiGlu>
+__device__ __forceinline__ void LoadActivations(const float* row, uint32_t at,
+                                                uint32_t cols, float (&v)[kValues]) {
+#pragma unroll
+  for (int q = 0; q < kValues / 4; ++q) {
+    float4 f = reinterpret_cast<const float4*>(row + at)[q];
+    if (kSwiGlu) {
+      const float4 u = reinterpret_cast<const float4*>(row + cols + at)[q];
+      f = make_float4(Silu(f.x) * u.x, Silu(f.y) * u.y, Silu(f.z) * u.z, Silu(f.w) * u.w);
+    }
+    v[4 * q + 0] = f.x;
+    v[4 * q + 1] = f.y;
+    v[4 * q + 2] = f.z;
+    v[4 * q + 3] = f.w;
+  }
+}
+
+// Quantizes all token columns into LDS.  A thread takes 8 consecutive values; the two
+// (Q6_K, groups of 16) or four (Q4_K/Q5_K, groups of 32) neighbouring threads of a
+// scale group agree on its largest magnitude and on sum(X) through quad exchanges.
+// The number of 8-value pieces per token is a multiple of 32, so quads are never
+// split by the loop bound.
 template <int TYPE, int NTOK, bool kSwiGlu>
-__device__ __forceinline__ void GemvBody(const GemvParams& prm,
-                                         const Columns<NTOK>& col,
-                                         const size_t* part_shift, float* lds) {
-  constexpr int kBlockBytes = BlockBytes(TYPE);
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int bpp_log2 = static_cast<int>(prm.bpp_log2);
-  const int bpp = 1 << bpp_log2;
-  const int rpp = 8 >> bpp_log2;
-  const int sub = lane & 7;
-  const int blk_lane = (lane >> 3) & (bpp - 1);
-  const int row_lane = lane >> (3 + bpp_log2);
-  const int lanes_per_row = 8 << bpp_log2;
-
-  const uint32_t nb = prm.launch.blocks_per_row;
-  const uint32_t chunk = prm.chunk_blocks;
-  const int x_stride = static_cast<int>(chunk) * 256;
-  const int s_stride = static_cast<int>(chunk) * 32;
-  float* lds_x = lds;
-  float* lds_s = lds + NTOK * x_stride;
-
-  // The rows this lane works on, one per visit.
-  const uint8_t* row_ptr[kVisits];
-  uint32_t y_index[kVisits];
-  bool valid[kVisits];
-  const uint32_t wg_row0 = blockIdx.x * prm.rows_per_wg;
+__device__ __forceinline__ void StageActivations(const GemvParams& prm,
+                                                 const Columns<NTOK>& col, U32x4* lds) {
+  constexpr bool kSix = TYPE == kTypeQ6K;
+  constexpr uint32_t kSlots = Slots<TYPE>();
+  const uint32_t bpp_log2 = prm.bpp_log2;
+  const uint32_t positions = 4u << bpp_log2;  // lanes that cover one pass of a row
+  const uint32_t octets = prm.launch.blocks_per_row * 32;  // 8-value pieces per token
+  for (uint32_t u = threadIdx.x; u < NTOK * octets; u += kThreads) {
+    const uint32_t t = u / octets;
+    const uint32_t o = u - t * octets;
+    const uint32_t block = o >> 5;
+    const uint32_t piece = o & 31;  // values 8*piece .. +8 of the block
+    float v[8];
+    LoadActivations<8, kSwiGlu>(ColumnX<NTOK>(col, t), block * 256 + piece * 8, prm.cols, v);
+    float gmax = 0.0f;
 #pragma unroll
-  for (int v = 0; v < kVisits; ++v) {
-    const uint32_t row = wg_row0 + (v * kWaves + wave) * rpp + row_lane;
-    uint32_t rest = row;
-    bool found = false;
-    row_ptr[v] = prm.launch.part[0].rows;
-    y_index[v] = 0;
+    for (int c = 0; c < 8; ++c) gmax = fmaxf(gmax, fabsf(v[c]));
+    gmax = fmaxf(gmax, __int_as_float(QuadSwap<0xB1>(__float_as_int(gmax))));
+    if (!kSix) gmax = fmaxf(gmax, __int_as_float(QuadSwap<0x4E>(__float_as_int(gmax))));
+    uint32_t limb[3][2];
+    float scale;
+    int sum;
+    QuantizeOctet(v, gmax, limb, &scale, &sum);
+    sum += QuadSwap<0xB1>(sum);
+    if (!kSix) sum += QuadSwap<0x4E>(sum);
+
+    const uint32_t pass = block >> bpp_log2;
+    const uint32_t blk_lane = block & ((1u << bpp_log2) - 1);
+    U32x4* base = lds + (static_cast<size_t>(t) * prm.passes + pass) * kSlots * positions +
+                  (blk_lane << 2);
+    if (kSix) {
+      // group = piece/2 = 8n + 2k + i; lane of the block = 2n + i.
+      const uint32_t group = piece >> 1;
+      const uint32_t half = piece & 1;  // first or second 8 of the 16
+      const uint32_t n = group >> 3;
+      const uint32_t k = (group & 7) >> 1;
+      const uint32_t i = group & 1;
+      base += 2 * n + i;
 #pragma unroll
-    for (int p = 0; p < kMaxGemvParts; ++p) {
-      if (p < static_cast<int>(prm.launch.n_parts) && !found) {
-        const GemvPart part = prm.launch.part[p];
-        if (rest < part.n_rows) {
-          row_ptr[v] = part.rows + (part_shift != nullptr ? part_shift[p] : 0) +
-                       static_cast<size_t>(rest) * prm.row_bytes;
-          y_index[v] = part.y_offset + rest;
-          found = true;
-        } else {
-          rest -= part.n_rows;
-        }
+      for (int l = 0; l < 3; ++l) {
+        U32x2* dst = reinterpret_cast<U32x2*>(base + (k * 3 + l) * positions) + half;
+        *dst = U32x2{limb[l][0], limb[l][1]};
       }
-    }
-    valid[v] = found && row < prm.launch.total_rows;
-  }
-
-  float acc[kVisits][NTOK];
-#pragma unroll
-  for (int v = 0; v < kVisits; ++v) {
-#pragma unroll
-    for (int t = 0; t < NTOK; ++t) acc[v][t] = 0.0f;
-  }
-
-  for (uint32_t c0 = 0; c0 < nb; c0 += chunk) {
-    const uint32_t cb = min(chunk, nb - c0);
-    if (c0 != 0) __syncthreads();
-    // Stage x[t][c0*256 .. (c0+cb)*256) and the sums of every 8 values.
-    const uint32_t units = cb * 32;  // groups of 8 values per token
-    for (uint32_t u = tid; u < NTOK * units; u += kThreads) {
-      const uint32_t t = u / units;
-      const uint32_t g = u - t * units;
-      const float4* src =
-          reinterpret_cast<const float4*>(col.x[t] + static_cast<size_t>(c0) * 256 + g * 8);
-      float4 v0 = src[0];
-      float4 v1 = src[1];
-      if (kSwiGlu) {
-        const float4* up = reinterpret_cast<const float4*>(
-            col.x[t] + prm.cols + static_cast<size_t>(c0) * 256 + g * 8);
-        const float4 u0 = up[0];
-        const float4 u1 = up[1];
-        v0 = make_float4(Silu(v0.x) * u0.x, Silu(v0.y) * u0.y, Silu(v0.z) * u0.z,
-                         Silu(v0.w) * u0.w);
-        v1 = make_float4(Silu(v1.x) * u1.x, Silu(v1.y) * u1.y, Silu(v1.z) * u1.z,
-                         Silu(v1.w) * u1.w);
+      if (half == 0) {
+        reinterpret_cast<float*>(base + 12 * positions)[k] = scale;
+        reinterpret_cast<int*>(base + 13 * positions)[k] = 32 * sum;
       }
-      float4* dst = reinterpret_cast<float4*>(lds_x + t * x_stride + g * 8);
-      dst[0] = v0;
-      dst[1] = v1;
-      lds_s[t * s_stride + g] =
-          ((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w));
-    }
-    __syncthreads();
-
-    const uint32_t passes = cb >> bpp_log2;
+    } else {
+      // sub-block j = piece/4; lane of the block = j/2, low or high nibbles = j%2.
+      const uint32_t j = piece >> 2;
+      const uint32_t quarter = piece & 3;  // which 8 of the 32
+      const uint32_t nibble = j & 1;
+      base += j >> 1;
 #pragma unroll
-    for (int v = 0; v < kVisits; ++v) {
-      if (!valid[v]) continue;
-      const uint8_t* base =
-          row_ptr[v] + static_cast<size_t>(c0 + blk_lane) * kBlockBytes;
-      for (uint32_t it = 0; it < passes; ++it) {
-        const uint32_t b = it * bpp + blk_lane;  // block within the chunk
-        MacBlock<TYPE, NTOK>(base + static_cast<size_t>(it) * bpp * kBlockBytes, sub,
-                             lds_x + b * 256, lds_s + b * 32, x_stride, s_stride,
-                             acc[v]);
+      for (int l = 0; l < 3; ++l) {
+        const uint32_t slot = (nibble * 3 + l) * 2 + (quarter >> 1);
+        U32x2* dst = reinterpret_cast<U32x2*>(base + slot * positions) + (quarter & 1);
+        *dst = U32x2{limb[l][0], limb[l][1]};
       }
-    }
-  }
-
-#pragma unroll
-  for (int v = 0; v < kVisits; ++v) {
-#pragma unroll
-    for (int t = 0; t < NTOK; ++t) {
-      const float total = GroupSum(acc[v][t], lanes_per_row);
-      if (valid[v] && (lane & (lanes_per_row - 1)) == 0) {
-        col.y[t][y_index[v]] = total;
+      if (quarter == 0) {
+        float* tail = reinterpret_cast<float*>(base + 12 * positions);
+        tail[nibble] = scale;
+        tail[2 + nibble] = scale * static_cast<float>(sum);
       }
     }
   }
 }
 
-// Dense product: token t reads x + t*cols and writes y + t*y_stride.
+__device__ __forceinline__ void LoadX(const U32x4* base, uint32_t positions, XK4* x) {
+#pragma unroll
+  for (int s = 0; s < 12; ++s) {
+    const U32x4 v = base[s * positions];
+    const int hl = s >> 1;  // half * 3 + limb
+    const int w0 = 4 * (s & 1);
+    x->limb[hl / 3][hl % 3][w0 + 0] = v.x;
+    x->limb[hl / 3][hl % 3][w0 + 1] = v.y;
+    x->limb[hl / 3][hl % 3][w0 + 2] = v.z;
+    x->limb[hl / 3][hl % 3][w0 + 3] = v.w;
+  }
+  const U32x4 tail = base[12 * positions];
+  x->xs[0] = __uint_as_float(tail.x);
+  x->xs[1] = __uint_as_float(tail.y);
+  x->fx[0] = __uint_as_float(tail.z);
+  x->fx[1] = __uint_as_float(tail.w);
+}
+
+__device__ __forceinline__ void LoadX(const U32x4* base, uint32_t positions, XQ6* x) {
+#pragma unroll
+  for (int s = 0; s < 12; ++s) {
+    const U32x4 v = base[s * positions];
+    x->limb[s / 3][s % 3][0] = v.x;
+    x->limb[s / 3][s % 3][1] = v.y;
+    x->limb[s / 3][s % 3][2] = v.z;
+    x->limb[s / 3][s % 3][3] = v.w;
+  }
+  const U32x4 scales = base[12 * positions];
+  const U32x4 sums = base[13 * positions];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    x->xs[k] = __uint_as_float(scales[k]);
+    x->sx32[k] = static_cast<int>(sums[k]);
+  }
+}
+
+// sum over 4*kWords values of code * X, exact: the limbs from the most significant
+// down, the accumulator shifted one byte between them.
+template <int kWords>
+__device__ __forceinline__ int CodeDot(const uint32_t (&codes)[kWords],
+                                       const uint32_t (&limb)[3][kWords]) {
+  int acc = 0;
+#pragma unroll
+  for (int w = 0; w < kWords; ++w) acc = Dot4(codes[w], limb[2][w], acc);
+  acc <<= 8;
+#pragma unroll
+  for (int w = 0; w < kWords; ++w) acc = Dot4(codes[w], limb[1][w], acc);
+  acc <<= 8;
+#pragma unroll
+  for (int w = 0; w < kWords; ++w) acc = Dot4(codes[w], limb[0][w], acc);
+  return acc;
+}
+
+// ---- one lane's share of a super-block: raw bytes, decode, multiply-accumulate ---
+
+// Q4_K / Q5_K.  Lane p (0..3) takes the p-th run of 32 quant bytes: sub-block 2p in
+// the low nibbles, 2p+1 in the high nibbles; Q5_K adds bit 2p / 2p+1 of qh[l] as the
+// fifth bit.  weight = (d*sc_j)*q - (dmin*m_j), so a sub-block contributes
+// (d*sc_j) * sum(q*x) - (dmin*m_j) * sum(x).
+template <bool kFifthBit>
+struct RawK4 {
+  U32x4 header;  // d, dmin, 12 packed scale bytes
+  U32x4 qs[2];
+  U32x4 qh[2];
+
+  __device__ __forceinline__ void Load(const uint8_t* blk, int lane4) {
+    header = Load16(blk);
+    const uint8_t* run = blk + 16 + (kFifthBit ? 32 : 0) + 32 * lane4;
+    qs[0] = Load16(run);
+    qs[1] = Load16(run + 16);
+    if (kFifthBit) {
+      qh[0] = Load16(blk + 16);
+      qh[1] = Load16(blk + 32);
+    }
+  }
+
+  template <int NTOK>
+  __device__ __forceinline__ void Mac(int lane4, const XK4 (&x)[NTOK],
+                                      float (&acc)[NTOK]) const {
+    const int p = lane4;
+    const float d = HalfBitsToFloat(header.x & 0xFFFFu);
+    const float dmin = HalfBitsToFloat(header.x >> 16);
+    uint32_t sc0, m0, sc1, m1;
+    ScaleMinK4(header.y, header.z, header.w, 2 * p, &sc0, &m0);
+    ScaleMinK4(header.y, header.z, header.w, 2 * p + 1, &sc1, &m1);
+    const float scale0 = d * static_cast<float>(sc0);
+    const float scale1 = d * static_cast<float>(sc1);
+    const float min0 = dmin * static_cast<float>(m0);
+    const float min1 = dmin * static_cast<float>(m1);
+    uint32_t lo[8];
+    uint32_t hi[8];
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const uint32_t q = qs[w >> 2][w & 3];
+      lo[w] = q & 0x0F0F0F0Fu;
+      hi[w] = (q >> 4) & 0x0F0F0F0Fu;
+      if (kFifthBit) {
+        const uint32_t h = qh[w >> 2][w & 3];
+        lo[w] |= ((h >> (2 * p)) & 0x01010101u) << 4;
+        hi[w] |= ((h >> (2 * p + 1)) & 0x01010101u) << 4;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+      const float dot_lo = static_cast<float>(CodeDot<8>(lo, x[t].limb[0])) * x[t].xs[0];
+      const float dot_hi = static_cast<float>(CodeDot<8>(hi, x[t].limb[1])) * x[t].xs[1];
+      float part = scale0 * dot_lo;
+      part = Fma(-min0, x[t].fx[0], part);
+      part = Fma(scale1, dot_hi, part);
+      part = Fma(-min1, x[t].fx[1], part);
+      acc[t] += part;
+    }
+  }
+};
+
+// Q6_K.  Lane (n, i) = (lane/2, lane%2) reads ql[64n+16i..+16), ql[64n+32+16i..+16)
+// and qh[32n+16i..+16) and so owns values 128n + 32k + 16i + c for k < 4, c < 16:
+// code = 4 low bits from the first (k even) or second (k odd) ql run, low nibble for
+// k < 2 and high nibble otherwise, plus bits 2k..2k+1 of qh.
+// weight = d * sc[8n + 2k + i] * (code - 32).
+struct RawQ6 {
+  U32x4 a;
+  U32x4 b;
+  U32x4 h;
+  U32x2 scales;  // this half's eight int8 scales
+  uint32_t d;
+
+  __device__ __forceinline__ void Load(const uint8_t* blk, int lane4) {
+    const int n = lane4 >> 1;
+    const int i = lane4 & 1;
+    a = Load16Align2(blk + 64 * n + 16 * i);
+    b = Load16Align2(blk + 64 * n + 32 + 16 * i);
+    h = Load16Align2(blk + 128 + 32 * n + 16 * i);
+    scales = Load8Align2(blk + 192 + 8 * n);
+    d = Load2(blk + 208);
+  }
+
+  template <int NTOK>
+  __device__ __forceinline__ void Mac(int lane4, const XQ6 (&x)[NTOK],
+                                      float (&acc)[NTOK]) const {
+    const int i = lane4 & 1;
+    uint32_t codes[4][4];
+    float scale[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      codes[0][w] = (a[w] & 0x0F0F0F0Fu) | ((h[w] << 4) & 0x30303030u);
+      codes[1][w] = (b[w] & 0x0F0F0F0Fu) | ((h[w] << 2) & 0x30303030u);
+      codes[2][w] = ((a[w] >> 4) & 0x0F0F0F0Fu) | (h[w] & 0x30303030u);
+      codes[3][w] = ((b[w] >> 4) & 0x0F0F0F0Fu) | ((h[w] >> 2) & 0x30303030u);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t word = k < 2 ? scales.x : scales.y;
+      const uint32_t shift = 8 * (((2 * k) & 3) + i);
+      scale[k] = static_cast<float>(static_cast<int>(word << (24u - shift)) >> 24);
+    }
+    const float df = HalfBitsToFloat(d);
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+      float block = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int dot = CodeDot<4>(codes[k], x[t].limb[k]) - x[t].sx32[k];
+        block = Fma(scale[k], static_cast<float>(dot) * x[t].xs[k], block);
+      }
+      acc[t] = Fma(df, block, acc[t]);
+    }
+  }
+};
+
+template <int TYPE>
+struct RawOf {
+  using Type = RawK4<TYPE == kTypeQ5K>;
+};
+template <>
+struct RawOf<kTypeQ6K> {
+  using Type = RawQ6;
+};
+
+// ---- cross-lane sum ----------------------------------------------------------------
+// Sum over a group of `lanes` (4..64, a power of two) consecutive lanes with DPP adds
+// in a fixed order.  The group's last lane ends with the total.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float DppAdd(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xF,
+                                                false);
+  return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float GroupTotal(float v, int lanes) {
+  v = DppAdd<0xB1, 0xF>(v);                    // quad_perm [1,0,3,2]
+  v = DppAdd<0x4E, 0xF>(v);                    // quad_perm [2,3,0,1]
+  if (lanes >= 8) v = DppAdd<0x141, 0xF>(v);   // row_half_mirror
+  if (lanes >= 16) v = DppAdd<0x140, 0xF>(v);  // row_mirror
+  if (lanes >= 32) v = DppAdd<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  if (lanes >= 64) v = DppAdd<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+  return v;
+}
+
+// ---- the product ---------------------------------------------------------------------
+
+// One workgroup's share.  Row group g (16 >> bpp_log2 consecutive flat rows) is
+// visited by one wave; this wave takes groups g_first, g_first + g_stride, ... below
+// g_end.  part_shift[p] (optional) is added to part p's row pointer: the byte offset
+// of an expert inside a 3-D tensor.
+template <int TYPE, int NTOK, bool kSwiGlu>
+__device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NTOK>& col,
+                                         const size_t* part_shift, uint32_t g_first,
+                                         uint32_t g_stride, uint32_t g_end, U32x4* lds) {
+  using Raw = typename RawOf<TYPE>::Type;
+  using X = typename XOf<TYPE>::Type;
+  constexpr int kBlockBytes = BlockBytes(TYPE);
+  constexpr uint32_t kSlots = Slots<TYPE>();
+
+  const int lane = threadIdx.x & 63;
+  const uint32_t bpp_log2 = prm.bpp_log2;
+  const uint32_t bpp = 1u << bpp_log2;
+  const uint32_t rpp = kBlocksPerPass >> bpp_log2;
+  const int lanes_per_row = 4 << bpp_log2;
+  const int lane4 = lane & 3;
+  const uint32_t blk_lane = (lane >> 2) & (bpp - 1);
+  const uint32_t row_lane = lane >> (2 + bpp_log2);
+  const uint32_t position = (blk_lane << 2) + lane4;
+  const uint32_t positions = 4u << bpp_log2;
+  const uint32_t passes = prm.passes;
+
+  // State of the kDepth visits in flight: where the lane's row starts, where its
+  // output goes, and the raw bytes of the next block to consume.
+  Raw raw[kDepth];
+  const uint8_t* row_base[kDepth];
+  uint32_t y_index[kDepth];
+  bool valid[kDepth];
+
+  const size_t shift0 = part_shift != nullptr ? part_shift[0] : 0;
+  const uint8_t* const base0 =
+      prm.launch.part[0].rows + shift0 + static_cast<size_t>(blk_lane) * kBlockBytes;
+  const uint32_t y_offset0 = prm.launch.part[0].y_offset;
+  const bool one_part = prm.launch.n_parts == 1;
+  auto locate = [&](int d, uint32_t group) {
+    const uint32_t flat = group * rpp + row_lane;
+    valid[d] = group < g_end && flat < prm.launch.total_rows;
+    if (one_part) {
+      row_base[d] = base0 + static_cast<size_t>(flat) * prm.row_bytes;
+      y_index[d] = y_offset0 + flat;
+      return;
+    }
+    const uint8_t* base = prm.launch.part[0].rows;
+    size_t shift = shift0;
+    uint32_t start = 0;
+    uint32_t y_offset = y_offset0;
+#pragma unroll
+    for (int p = 1; p < kMaxGemvParts; ++p) {
+      if (p < static_cast<int>(prm.launch.n_parts) && flat >= prm.start[p]) {
+        base = prm.launch.part[p].rows;
+        shift = part_shift != nullptr ? part_shift[p] : 0;
+        start = prm.start[p];
+        y_offset = prm.launch.part[p].y_offset;
+      }
+    }
+    row_base[d] = base + shift + static_cast<size_t>(flat - start) * prm.row_bytes +
+                  static_cast<size_t>(blk_lane) * kBlockBytes;
+    y_index[d] = y_offset + (flat - start);
+  };
+  auto issue = [&](int d, uint32_t pass) {
+    if (valid[d]) {
+      raw[d].Load(row_base[d] + static_cast<size_t>(pass) * bpp * kBlockBytes, lane4);
+    }
+  };
+
+  // Weight loads first, so that their latency overlaps the staging of x.
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) {
+    locate(d, g_first + d * g_stride);
+    issue(d, 0);
+  }
+
+  StageActivations<TYPE, NTOK, kSwiGlu>(prm, col, lds);
+  __syncthreads();
+
+  X x[NTOK];
+  float acc[kDepth][NTOK];
+  uint32_t group0 = g_first;  // group of visit 0 of the current iteration
+  uint32_t pass = 0;
+  while (group0 < g_end) {
+    if (pass == 0) {
+#pragma unroll
+      for (int d = 0; d < kDepth; ++d) {
+#pragma unroll
+        for (int t = 0; t < NTOK; ++t) acc[d][t] = 0.0f;
+      }
+    }
+    if (passes > 1 || group0 == g_first) {
+#pragma unroll
+      for (int t = 0; t < NTOK; ++t) {
+        LoadX(lds + (static_cast<size_t>(t) * passes + pass) * kSlots * positions + position,
+              positions, &x[t]);
+      }
+    }
+    const bool last_pass = pass + 1 == passes;
+    const uint32_t next_pass = last_pass ? 0 : pass + 1;
+    const uint32_t next_group0 = last_pass ? group0 + kDepth * g_stride : group0;
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      // The arithmetic of this visit, then the loads of the visit that takes over its
+      // registers: kDepth - 1 visits stay in flight meanwhile.
+      if (valid[d]) raw[d].Mac(lane4, x, acc[d]);
+      if (last_pass) {
+#pragma unroll
+        for (int t = 0; t < NTOK; ++t) {
+          const float total = GroupTotal(acc[d][t], lanes_per_row);
+          if (valid[d] && (lane & (lanes_per_row - 1)) == lanes_per_row - 1) {
+            col.y[t][y_index[d]] = total;
+          }
+        }
+        locate(d, next_group0 + d * g_stride);
+      }
+      issue(d, next_pass);
+    }
+    pass = next_pass;
+    group0 = next_group0;
+  }
+}
+
+// Dense product: token t reads x + t*cols and writes y + t*y_stride; the waves of
+// the whole grid share the row groups round robin.
 template <int TYPE, int NTOK>
 __global__ __launch_bounds__(kThreads) void KquantGemvKernel(
     const GemvParams prm, const float* __restrict__ x, float* __restrict__ y) {
-  extern __shared__ __align__(16) float lds[];
+  extern __shared__ __align__(16) U32x4 lds[];
   Columns<NTOK> col;
 #pragma unroll
   for (int t = 0; t < NTOK; ++t) {
     col.x[t] = x + static_cast<size_t>(t) * prm.cols;
     col.y[t] = y + static_cast<size_t>(t) * prm.launch.y_stride;
   }
-  GemvBody<TYPE, NTOK, false>(prm, col, nullptr, lds);
+  const uint32_t wave = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  GemvBody<TYPE, NTOK, false>(prm, col, nullptr, wave, gridDim.x * kWavesPerGroup,
+                              prm.n_groups, lds);
 }
 
-// Expert product: blockIdx.y names a segment, i.e. one routed expert and up to
-// four of the (token, slot) pairs that chose it.  The expert's rows are streamed
-// once for all of them.  Column t reads the activation row of its pair (the
-// token's x, or with kSwiGlu the pair's [gate | up] row) and writes the pair's
-// output row.
+// Expert product: blockIdx.y names a segment, i.e. one routed expert and up to four
+// of the (token, slot) pairs that chose it; blockIdx.x a tile of the expert's row
+// groups.  The expert's rows are streamed once for all of the segment's pairs.
+// Column t reads the activation row of its pair (the token's x, or with kSwiGlu the
+// pair's [gate | up] row) and writes the pair's output row.
 template <int TYPE, int NTOK, bool kSwiGlu>
 __device__ __forceinline__ void MoeSegmentBody(const GemvParams& prm,
                                                const MoeGemvArgs& moe,
-                                               const MoeSegment& seg, float* lds) {
+                                               const MoeSegment& seg, U32x4* lds) {
   Columns<NTOK> col;
 #pragma unroll
   for (int t = 0; t < NTOK; ++t) {
@@ -352,13 +630,17 @@ __device__ __forceinline__ void MoeSegmentBody(const GemvParams& prm,
   for (int p = 0; p < kMaxGemvParts; ++p) {
     shift[p] = static_cast<size_t>(seg.expert) * moe.expert_bytes[p];
   }
-  GemvBody<TYPE, NTOK, kSwiGlu>(prm, col, shift, lds);
+  const uint32_t groups_per_tile = kWavesPerGroup * kDepth;
+  const uint32_t first = blockIdx.x * groups_per_tile;
+  const uint32_t end = min(first + groups_per_tile, prm.n_groups);
+  GemvBody<TYPE, NTOK, kSwiGlu>(prm, col, shift, first + (threadIdx.x >> 6),
+                                kWavesPerGroup, end, lds);
 }
 
 template <int TYPE, bool kSwiGlu>
 __global__ __launch_bounds__(kThreads) void KquantMoeGemvKernel(const GemvParams prm,
                                                                 const MoeGemvArgs moe) {
-  extern __shared__ __align__(16) float lds[];
+  extern __shared__ __align__(16) U32x4 lds[];
   const uint32_t s = blockIdx.y;
   if (s >= static_cast<uint32_t>(moe.tables->n_segments)) return;
   const MoeSegment seg = moe.segments[s];
@@ -370,49 +652,11 @@ __global__ __launch_bounds__(kThreads) void KquantMoeGemvKernel(const GemvParams
   }
 }
 
-template <int TYPE>
-hipError_t LaunchTyped(const GemvParams& prm, const float* x, int tokens, float* y,
-                       dim3 grid, size_t lds_bytes, hipStream_t stream) {
-  switch (tokens) {
-    case 1:
-      hipLaunchKernelGGL((KquantGemvKernel<TYPE, 1>), grid, dim3(kThreads), lds_bytes,
-                         stream, prm, x, y);
-      break;
-    case 2:
-      hipLaunchKernelGGL((KquantGemvKernel<TYPE, 2>), grid, dim3(kThreads), lds_bytes,
-                         stream, prm, x, y);
-      break;
-    case 3:
-      hipLaunchKernelGGL((KquantGemvKernel<TYPE, 3>), grid, dim3(kThreads), lds_bytes,
-                         stream, prm, x, y);
-      break;
-    case 4:
-      hipLaunchKernelGGL((KquantGemvKernel<TYPE, 4>), grid, dim3(kThreads), lds_bytes,
-                         stream, prm, x, y);
-      break;
-    default:
-      return hipErrorInvalidValue;
-  }
-  return hipGetLastError();
-}
+// ---- host side -------------------------------------------------------------------------
 
-// Fills the launch geometry for `tokens` columns; returns the dynamic LDS bytes.
-size_t PlanGemv(int type, const GemvLaunch& launch, int tokens, GemvParams* prm) {
-  prm->launch = launch;
-  const uint32_t nb = launch.blocks_per_row;
-  prm->row_bytes = nb * BlockBytes(type);
-  prm->cols = nb * 256;
-  uint32_t bpp_log2 = 0;
-  while (bpp_log2 < 3 && (nb & ((2u << bpp_log2) - 1)) == 0) ++bpp_log2;
-  prm->bpp_log2 = bpp_log2;
-  prm->rows_per_wg = kVisits * kWaves * (8u >> bpp_log2);
-  // As many super-blocks of x per chunk as the LDS budget holds, in multiples of
-  // 8 (every bpp divides 8), or the whole row when it fits.
-  uint32_t chunk = kLdsBudget / (tokens * kLdsFloatsPerBlock * 4);
-  chunk = chunk / 8 * 8;
-  if (chunk >= nb) chunk = nb;
-  prm->chunk_blocks = chunk;
-  return static_cast<size_t>(tokens) * chunk * kLdsFloatsPerBlock * sizeof(float);
+size_t LdsBytes(int type, uint32_t blocks_per_row, int tokens) {
+  const size_t slots = type == kTypeQ6K ? Slots<kTypeQ6K>() : Slots<kTypeQ4K>();
+  return static_cast<size_t>(tokens) * blocks_per_row * 4 * slots * 16;
 }
 
 bool ValidLaunch(int type, const GemvLaunch& launch) {
@@ -420,30 +664,95 @@ bool ValidLaunch(int type, const GemvLaunch& launch) {
          launch.n_parts <= kMaxGemvParts && launch.blocks_per_row != 0;
 }
 
+void PlanGemv(int type, const GemvLaunch& launch, GemvParams* prm) {
+  prm->launch = launch;
+  const uint32_t nb = launch.blocks_per_row;
+  prm->row_bytes = nb * BlockBytes(type);
+  prm->cols = nb * 256;
+  uint32_t bpp_log2 = 0;
+  while (bpp_log2 < 4 && (nb & ((2u << bpp_log2) - 1)) == 0) ++bpp_log2;
+  prm->bpp_log2 = bpp_log2;
+  prm->passes = nb >> bpp_log2;
+  const uint32_t rpp = kBlocksPerPass >> bpp_log2;
+  prm->n_groups = (launch.total_rows + rpp - 1) / rpp;
+  uint32_t start = 0;
+  for (uint32_t p = 0; p < static_cast<uint32_t>(kMaxGemvParts); ++p) {
+    prm->start[p] = start;
+    if (p < launch.n_parts) start += launch.part[p].n_rows;
+  }
+}
+
+// Kernels whose LDS need may exceed the 64 KB default are allowed the full LDS of a
+// gfx950 compute unit.
+template <typename Kernel>
+hipError_t AllowLargeLds(Kernel kernel, size_t lds_bytes) {
+  if (lds_bytes <= 64 * 1024) return hipSuccess;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                             static_cast<int>(kGemvMaxLdsBytes));
+}
+
+template <int TYPE, int NTOK>
+hipError_t LaunchDense(const GemvParams& prm, const float* x, float* y, dim3 grid,
+                       size_t lds_bytes, hipStream_t stream) {
+  const hipError_t status = AllowLargeLds(KquantGemvKernel<TYPE, NTOK>, lds_bytes);
+  if (status != hipSuccess) return status;
+  hipLaunchKernelGGL((KquantGemvKernel<TYPE, NTOK>), grid, dim3(kThreads), lds_bytes, stream,
+                     prm, x, y);
+  return hipGetLastError();
+}
+
+template <int TYPE>
+hipError_t LaunchTyped(const GemvParams& prm, const float* x, int tokens, float* y,
+                       dim3 grid, size_t lds_bytes, hipStream_t stream) {
+  switch (tokens) {
+    case 1: return LaunchDense<TYPE, 1>(prm, x, y, grid, lds_bytes, stream);
+    case 2: return LaunchDense<TYPE, 2>(prm, x, y, grid, lds_bytes, stream);
+    case 3: return LaunchDense<TYPE, 3>(prm, x, y, grid, lds_bytes, stream);
+    case 4: return LaunchDense<TYPE, 4>(prm, x, y, grid, lds_bytes, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int TYPE>
 hipError_t LaunchMoeTyped(const GemvParams& prm, const MoeGemvArgs& moe, bool swiglu,
                           dim3 grid, size_t lds_bytes, hipStream_t stream) {
   if (swiglu) {
-    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, true>), grid, dim3(kThreads),
-                       lds_bytes, stream, prm, moe);
+    const hipError_t status = AllowLargeLds(KquantMoeGemvKernel<TYPE, true>, lds_bytes);
+    if (status != hipSuccess) return status;
+    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, true>), grid, dim3(kThreads), lds_bytes,
+                       stream, prm, moe);
   } else {
-    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, false>), grid, dim3(kThreads),
-                       lds_bytes, stream, prm, moe);
+    const hipError_t status = AllowLargeLds(KquantMoeGemvKernel<TYPE, false>, lds_bytes);
+    if (status != hipSuccess) return status;
+    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, false>), grid, dim3(kThreads), lds_bytes,
+                       stream, prm, moe);
   }
   return hipGetLastError();
 }
 
 }  // namespace
 
+int GemvMaxTokens(int type, uint32_t blocks_per_row) {
+  const size_t per_token = LdsBytes(type, blocks_per_row, 1);
+  if (per_token == 0) return 0;
+  const size_t fit = kGemvMaxLdsBytes / per_token;
+  return static_cast<int>(fit < static_cast<size_t>(kMaxGemvTokens) ? fit : kMaxGemvTokens);
+}
+
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream) {
-  if (!ValidLaunch(type, launch) || tokens < 1 || tokens > kMaxGemvTokens) {
+  if (!ValidLaunch(type, launch) || tokens < 1 ||
+      tokens > GemvMaxTokens(type, launch.blocks_per_row)) {
     return hipErrorInvalidValue;
   }
   if (launch.total_rows == 0) return hipSuccess;
   GemvParams prm;
-  const size_t lds_bytes = PlanGemv(type, launch, tokens, &prm);
-  const dim3 grid((launch.total_rows + prm.rows_per_wg - 1) / prm.rows_per_wg);
+  PlanGemv(type, launch, &prm);
+  const size_t lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens);
+  uint32_t blocks = (prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
+  if (blocks > kMaxGrid) blocks = kMaxGrid;
+  const dim3 grid(blocks);
   switch (type) {
     case kTypeQ4K: return LaunchTyped<kTypeQ4K>(prm, x, tokens, y, grid, lds_bytes, stream);
     case kTypeQ5K: return LaunchTyped<kTypeQ5K>(prm, x, tokens, y, grid, lds_bytes, stream);
@@ -453,13 +762,17 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
 
 hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& moe,
                          bool swiglu, uint32_t max_segments, hipStream_t stream) {
-  if (!ValidLaunch(type, launch)) return hipErrorInvalidValue;
+  if (!ValidLaunch(type, launch) ||
+      GemvMaxTokens(type, launch.blocks_per_row) < kMaxGemvTokens) {
+    return hipErrorInvalidValue;
+  }
   if (launch.total_rows == 0 || max_segments == 0) return hipSuccess;
   GemvParams prm;
+  PlanGemv(type, launch, &prm);
   // Sized for the widest segment (four columns); narrower ones use less of it.
-  const size_t lds_bytes = PlanGemv(type, launch, kMaxGemvTokens, &prm);
-  const dim3 grid((launch.total_rows + prm.rows_per_wg - 1) / prm.rows_per_wg,
-                  max_segments);
+  const size_t lds_bytes = LdsBytes(type, launch.blocks_per_row, kMaxGemvTokens);
+  const uint32_t groups_per_tile = kWavesPerGroup * kDepth;
+  const dim3 grid((prm.n_groups + groups_per_tile - 1) / groups_per_tile, max_segments);
   switch (type) {
     case kTypeQ4K: return LaunchMoeTyped<kTypeQ4K>(prm, moe, swiglu, grid, lds_bytes, stream);
     case kTypeQ5K: return LaunchMoeTyped<kTypeQ5K>(prm, moe, swiglu, grid, lds_bytes, stream);

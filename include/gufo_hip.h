@@ -202,9 +202,10 @@ int gufo_hip_graph_destroy(gufo_hip_graph* graph);
  * the stop event, waits for it and returns the milliseconds between them. */
 int gufo_hip_timer_begin(void);
 int gufo_hip_timer_end(float* milliseconds);
-/* A plain streaming read of `bytes` of device memory (sum of dwords written to
- * *sink_dev): the achievable-read-bandwidth probe, as the reference measures its
- * own ceiling (src/npu/device.hpp:58-74). */
+/* A plain streaming read of `bytes` of device memory: the achievable-read-bandwidth
+ * probe, as the reference measures its own ceiling (src/npu/device.hpp:58-74).
+ * *sink_dev is written only if a lane's xor of its data equals a magic constant
+ * (that keeps the loads alive without timing a store). */
 int gufo_hip_read_probe_dev(const void* src_dev, size_t bytes, uint32_t* sink_dev);
 
 #ifdef __cplusplus
