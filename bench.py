@@ -109,6 +109,129 @@ def time_calls(capi, call, steps, warmup):
     return ms / steps
 
 
+def time_recorded(capi, calls, reps=20, warmup=3):
+    """Per-call time of `calls` (a list of thunks that enqueue _dev products):
+    recorded once as one graph and replayed, so host enqueue cost stays out."""
+    for call in calls:  # an ordinary pass first: recording cannot allocate scratch
+        call()
+    capi.synchronize()
+    capi.capture_begin()
+    for call in calls:
+        call()
+    graph = capi.capture_end()
+    for _ in range(warmup):
+        graph.launch()
+    capi.synchronize()
+    capi.timer_begin()
+    for _ in range(reps):
+        graph.launch()
+    ms = capi.timer_end()
+    capi.synchronize()
+    graph.destroy()
+    return ms / (reps * len(calls))
+
+
+def report(name, nbytes, ms, extra=""):
+    log(f"  {name:34s} {nbytes / 1e6:8.2f} MB  {ms * 1e3:8.2f} us  {nbytes / ms / 1e6:8.1f} GB/s"
+        f"  {100 * nbytes / ms / 1e6 / HBM_PEAK_GBS:5.1f}% of peak {extra}")
+
+
+def run_details(capi, cfg, synth, decode, args):
+    """Every stage of the decode set and the other measured configurations, each
+    rotating over enough weight copies to stay out of the 256 MB last-level cache."""
+    import numpy as np
+
+    log("config 2, per stage (N=1):")
+    for stage, names in cfg.CONFIG2_STAGES.items():
+        nbytes = sum(cfg.CONFIG2[n].nbytes for n in names)
+        n = 6 if stage == "lm_head" else 30
+        ms = time_recorded(capi, [lambda i=i, s=stage: decode.stage(s, i) for i in range(n)])
+        report(stage, nbytes, ms)
+
+    log("read probe (plain streaming read, the ceiling a kernel can reach):")
+    probe = capi.DeviceBuffer(1 << 30)
+    sink = capi.DeviceBuffer(64)
+    window = 256 << 20
+    ms = time_recorded(capi, [lambda i=i: capi.read_probe_dev_at(probe, (i % 4) * window, window,
+                                                                 sink) for i in range(8)])
+    report("read probe 256 MiB", window, ms)
+    probe.free()
+
+    log("config 1, single Q4_K GEMV 6144x2048 (N=1), 40 weight copies:")
+    spec = cfg.CONFIG1
+    host = spec.build()
+    mats = [capi.Matrix(spec.ggml_type, host, spec.rows, spec.cols) for _ in range(40)]
+    x = capi.DeviceBuffer.from_array(synth.activations(1, spec.cols, cfg.CONFIG1_X_SEED))
+    y = capi.DeviceBuffer(4 * spec.rows)
+    ms = time_recorded(capi, [lambda m=m: capi.gemv_dev([capi.whole(m)], x, 1, y) for m in mats])
+    report("q4_k 6144x2048 from HBM", spec.nbytes, ms)
+    ms = time_recorded(capi, [lambda: capi.gemv_dev([capi.whole(mats[0])], x, 1, y)] * 40)
+    report("q4_k 6144x2048 cache resident", spec.nbytes, ms)
+    for m in mats:
+        m.destroy()
+
+    log("config 3, MTP-verify FFN (gate|up 9216x2560 Q4_K, down 2560x9216 Q6_K), 8 copies:")
+    gate, up, down = (cfg.CONFIG3[n] for n in ("gate", "up", "down"))
+    hg, hu, hd = gate.build(), up.build(), down.build()
+    sets = [(capi.Matrix(gate.ggml_type, hg, gate.rows, gate.cols),
+             capi.Matrix(up.ggml_type, hu, up.rows, up.cols),
+             capi.Matrix(down.ggml_type, hd, down.rows, down.cols)) for _ in range(8)]
+    base = {}
+    for tokens in (1, 2, 3, 4):
+        xin = capi.DeviceBuffer.from_array(synth.activations(tokens, cfg.HIDDEN3, 1))
+        act = capi.DeviceBuffer.from_array(synth.activations(tokens, cfg.FFN3, 2))
+        y_in = capi.DeviceBuffer(4 * tokens * 2 * cfg.FFN3)
+        y_down = capi.DeviceBuffer(4 * tokens * cfg.HIDDEN3)
+        ms_in = time_recorded(capi, [lambda s=s: capi.gemv_dev([capi.whole(s[0]), capi.whole(s[1])],
+                                                               xin, tokens, y_in) for s in sets])
+        ms_down = time_recorded(capi, [lambda s=s: capi.gemv_dev([capi.whole(s[2])], act, tokens,
+                                                                 y_down) for s in sets])
+        if tokens == 1:
+            base = {"in": ms_in, "down": ms_down}
+        report(f"gate|up N={tokens}", gate.nbytes + up.nbytes, ms_in,
+               f"x{ms_in / base['in']:.2f} of N=1")
+        report(f"down    N={tokens}", down.nbytes, ms_down, f"x{ms_down / base['down']:.2f} of N=1")
+        for b in (xin, act, y_in, y_down):
+            b.free()
+    for s in sets:
+        for m in s:
+            m.destroy()
+
+    log("config 4, MoE experts (256 experts, hidden 2048, ffn 512, top-8):")
+    gate, up, down = (cfg.CONFIG4[n] for n in ("gate", "up", "down"))
+    mg = capi.Matrix(gate.ggml_type, gate.build(), gate.rows, gate.cols)
+    mu = capi.Matrix(up.ggml_type, up.build(), up.rows, up.cols)
+    md = capi.Matrix(down.ggml_type, down.build(), down.rows, down.cols)
+    per_expert = (gate.nbytes + up.nbytes + down.nbytes) // cfg.EXPERTS4
+    for tokens in (1, 4):
+        calls, distinct = [], []
+        keep = []
+        for r in range(16):  # 16 different routings, so successive calls read other experts
+            logits = synth.router_logits(tokens, cfg.EXPERTS4, 900 + 16 * tokens + r)
+            xh = synth.activations(tokens, cfg.HIDDEN4, 950 + r) * np.float32(cfg.CONFIG4_X_SCALE)
+            dl = capi.DeviceBuffer.from_array(logits)
+            dx = capi.DeviceBuffer.from_array(xh)
+            ids = capi.DeviceBuffer(4 * tokens * cfg.TOPK4)
+            wts = capi.DeviceBuffer(4 * tokens * cfg.TOPK4)
+            yo = capi.DeviceBuffer(4 * tokens * cfg.HIDDEN4)
+            keep += [dl, dx, ids, wts, yo]
+            host_ids, _ = capi.route_topk(logits, cfg.TOPK4)
+            distinct.append(len(set(host_ids.reshape(-1).tolist())))
+
+            def call(dl=dl, dx=dx, ids=ids, wts=wts, yo=yo):
+                capi.route_topk_dev(dl, tokens, cfg.EXPERTS4, cfg.TOPK4, ids, wts)
+                capi.moe_ffn_dev(mg, mu, md, cfg.EXPERTS4, dx, tokens, ids, wts, cfg.TOPK4, yo)
+            calls.append(call)
+        ms = time_recorded(capi, calls)
+        mean_distinct = sum(distinct) / len(distinct)
+        report(f"route+group+experts batch {tokens}", int(mean_distinct * per_expert), ms,
+               f"({mean_distinct:.1f} distinct experts, 6 kernels)")
+        for b in keep:
+            b.free()
+    for m in (mg, mu, md):
+        m.destroy()
+
+
 def cpu_baseline(cfg, decode, seconds):
     """The same set on the host cores: the reference's fused AVX2 dots on its own
     thread pool (oracle/_ref), or the scalar C restatement where that is absent."""
@@ -224,11 +347,7 @@ def main():
     }
 
     if args.details:
-        for stage, names in cfg.CONFIG2_STAGES.items():
-            nbytes = sum(cfg.CONFIG2[n].nbytes for n in names)
-            ms = time_calls(capi, lambda i, s=stage: decode.stage(s, i), args.steps, args.warmup)
-            log(f"  {stage:13s} {nbytes / 1e6:8.2f} MB  {ms * 1e3:8.2f} us  "
-                f"{nbytes / ms / 1e6:8.1f} GB/s")
+        run_details(capi, cfg, synth, decode, args)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, decode, args.cpu_seconds)

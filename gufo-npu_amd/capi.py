@@ -15,7 +15,8 @@ from typing import Sequence
 import numpy as np
 
 PACKAGE_DIR = Path(__file__).resolve().parent
-LIBRARY_PATH = PACKAGE_DIR / "lib" / "libgufo_hip.so"
+# GUFO_HIP_LIBRARY names another build of the same library (kernel experiments).
+LIBRARY_PATH = Path(os.environ.get("GUFO_HIP_LIBRARY") or PACKAGE_DIR / "lib" / "libgufo_hip.so")
 
 OK = 0
 ERR_NO_DEVICE = 1
@@ -373,6 +374,14 @@ def timer_end() -> float:
     ms = C.c_float(0.0)
     _check(load_library().gufo_hip_timer_end(C.byref(ms)))
     return ms.value
+
+
+def read_probe_dev_at(src: DeviceBuffer, offset: int, nbytes: int, sink: DeviceBuffer) -> None:
+    """The read probe over src[offset : offset + nbytes] (offset a multiple of 16)."""
+    if offset % 16 or offset + nbytes > src.nbytes:
+        raise ValueError("probe window outside the buffer")
+    _check(load_library().gufo_hip_read_probe_dev(C.c_void_p(src.ptr + offset), nbytes,
+                                                  C.c_void_p(sink.ptr)))
 
 
 def read_probe_dev(src: DeviceBuffer, nbytes: int, sink: DeviceBuffer) -> None:

@@ -308,6 +308,8 @@ int GroupDevLocked(const int* ids, int tokens, int k, int experts,
   }
   GUFO_TRY(ReserveMoeTables(static_cast<int>(n_pairs > 0 ? n_pairs : 1), experts, tables));
   GUFO_HIP_TRY(gufo::LaunchMoeGroup(ids, static_cast<int>(n_pairs), experts,
+                                    tokens < kMaxGemvTokens ? (tokens > 0 ? tokens : 1)
+                                                            : kMaxGemvTokens,
                                     tables->counts, tables->offsets, tables->pairs,
                                     tables->valid, tables->segments, tables->header,
                                     g_state.stream));
@@ -348,6 +350,8 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   float* gate_up = static_cast<float*>(g_state.moe_gate_up.ptr);
   float* routed = static_cast<float*>(g_state.moe_out.ptr);
 
+  // The grouping kernel cuts segments at min(tokens, 4) pairs.
+  const int max_pairs = tokens < kMaxGemvTokens ? tokens : kMaxGemvTokens;
   gufo::MoeGemvArgs args;
   std::memset(&args, 0, sizeof args);
   args.tables = tables.header;
@@ -368,15 +372,16 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
       launch.part[count].rows = in_parts[p]->data;
       launch.part[count].n_rows = static_cast<uint32_t>(ffn);
       launch.part[count].y_offset = static_cast<uint32_t>(p * ffn);
-      args.expert_bytes[count] = ffn * in_parts[p]->row_bytes;
       ++count;
     }
+    args.expert_bytes = ffn * in_parts[first]->row_bytes;
     launch.n_parts = static_cast<uint32_t>(count);
     launch.total_rows = static_cast<uint32_t>(count * ffn);
     launch.blocks_per_row = static_cast<uint32_t>(hidden / gufo::kSuperBlock);
     launch.y_stride = static_cast<uint32_t>(2 * ffn);
     GUFO_HIP_TRY(gufo::LaunchMoeGemv(type, launch, args, false,
-                                     static_cast<uint32_t>(n_pairs), g_state.stream));
+                                     static_cast<uint32_t>(n_pairs), max_pairs,
+                                     g_state.stream));
     first += count;
   }
 
@@ -394,10 +399,10 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
     args.x = gate_up;
     args.x_row_floats = 2 * ffn;
     args.y = routed;
-    std::memset(args.expert_bytes, 0, sizeof args.expert_bytes);
-    args.expert_bytes[0] = hidden * down->row_bytes;
+    args.expert_bytes = hidden * down->row_bytes;
     GUFO_HIP_TRY(gufo::LaunchMoeGemv(down->type, launch, args, true,
-                                     static_cast<uint32_t>(n_pairs), g_state.stream));
+                                     static_cast<uint32_t>(n_pairs), max_pairs,
+                                     g_state.stream));
   }
   GUFO_HIP_TRY(gufo::LaunchMoeCombine(routed, weights, tables.valid, tokens, k,
                                       static_cast<int>(hidden), y, g_state.stream));
@@ -455,6 +460,7 @@ int gufo_hip_init(int device) {
   GUFO_HIP_TRY(hipEventCreate(&g_state.timer_end));
   std::snprintf(g_state.name, sizeof g_state.name, "%s (%s)", prop.gcnArchName, prop.name);
   g_state.compute_units = prop.multiProcessorCount;
+  gufo::SetGemvComputeUnits(prop.multiProcessorCount);
   g_state.device = device;
   g_state.ready = true;
   const int code = Reserve(&g_state.small, kSmallBytes);

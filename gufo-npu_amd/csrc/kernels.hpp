@@ -28,6 +28,9 @@ struct GemvLaunch {
 // LDS a product kernel may use: the whole LDS of a gfx950 compute unit.
 constexpr size_t kGemvMaxLdsBytes = 160 * 1024;
 
+// The compute-unit count of the device, which sizes the persistent launches.
+void SetGemvComputeUnits(int compute_units);
+
 // Token columns one launch can carry for rows of blocks_per_row super-blocks: the
 // quantized activation rows of all columns must fit in LDS together (at most
 // kMaxGemvTokens).
@@ -63,15 +66,17 @@ struct MoeGemvArgs {
   size_t x_row_floats;  // floats between activation rows
   float* y;             // output rows, one per pair, y_stride floats apart
   uint32_t k;           // slots per token
-  size_t expert_bytes[kMaxGemvParts];  // bytes between experts, per part
+  size_t expert_bytes;  // bytes between experts, the same for every part of a launch
 };
 
 // As LaunchGemv, once per segment: part p's rows start at
-// part[p].rows + segment.expert * expert_bytes[p].  swiglu = false: column t reads
+// part[p].rows + segment.expert * expert_bytes.  max_pairs bounds the pairs of a
+// segment (the call's token count, at most kMaxGemvTokens).  swiglu = false: column t reads
 // x row (pair / k); swiglu = true: column t reads the pair's own row of 2*cols
 // values [gate | up] and the product is taken with silu(gate) * up.
 hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& moe,
-                         bool swiglu, uint32_t max_segments, hipStream_t stream);
+                         bool swiglu, uint32_t max_segments, int max_pairs,
+                         hipStream_t stream);
 
 // Softmax (double) top-k routing of `tokens` rows of `experts` logits.
 constexpr int kMaxRouteExperts = 1024;
@@ -81,11 +86,12 @@ hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int*
 
 // Groups the n_pairs = tokens*k pairs by expert: counts[experts],
 // offsets[experts+1], pairs[n_pairs] (ascending pair id within an expert),
-// pair_valid[n_pairs], the segment list (at most n_pairs entries) and *tables.
+// pair_valid[n_pairs], the segment list (at most n_pairs entries, `capacity` pairs
+// each at most) and *tables.
 constexpr int kMaxGroupExperts = 1024;
 constexpr int kMaxGroupPairs = 8192;
-hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int* counts,
-                          int* offsets, int* pairs, uint8_t* pair_valid,
+hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int capacity,
+                          int* counts, int* offsets, int* pairs, uint8_t* pair_valid,
                           MoeSegment* segments, MoeTables* tables, hipStream_t stream);
 
 // y[t][i] = sum over slots in order of weights[t*k+slot] * rows[(t*k+slot)][i],

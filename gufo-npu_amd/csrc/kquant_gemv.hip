@@ -9,10 +9,11 @@
 // The kernel is bound by the HBM read of the packed weights, so everything else is
 // arranged to keep that stream saturated:
 //
-//   * Persistent waves.  A launch has at most a few workgroups per compute unit;
-//     every wave walks the rows in a grid-stride loop and keeps kDepth row visits
-//     of weight loads in flight in registers (issue the loads of visit i+kDepth,
-//     then do the arithmetic of visit i).
+//   * Persistent waves.  A launch has no more workgroups than are resident at once;
+//     every wave walks the rows in a grid-stride loop and holds two or three row
+//     visits of weight loads in registers: after the arithmetic of a visit its
+//     registers are reloaded with the visit that many steps ahead, so the other
+//     visits' loads are in flight during the arithmetic.
 //   * Four lanes per super-block, 64 weights per lane, 16 super-blocks per wave
 //     pass.  Each lane's share of a block is two or three 16-byte loads (Q6_K
 //     blocks are 210 bytes, so those loads are only 2-byte aligned, which gfx950
@@ -45,9 +46,29 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerGroup = kThreads / 64;
-constexpr int kDepth = 4;          // row visits of weight loads in flight per wave
 constexpr int kBlocksPerPass = 16;  // super-blocks a wave covers per pass (4 lanes each)
-constexpr uint32_t kMaxGrid = 512;  // persistent workgroups of a dense launch
+
+// Tuning, by token columns of the launch.  One column leaves registers for three
+// row visits of prefetched weights at three waves per SIMD, the occupancy the
+// 151,936-row lm_head measured fastest at; more columns hold more quantized
+// activations in registers, so they run at lower occupancy and shallower prefetch.
+// The macros are for kernel experiments (-D on the hipcc line).
+#ifndef GUFO_GEMV_DEPTH
+#define GUFO_GEMV_DEPTH 3
+#endif
+#ifndef GUFO_GEMV_WAVES_PER_EU
+#define GUFO_GEMV_WAVES_PER_EU 3
+#endif
+__host__ __device__ constexpr int DepthFor(int tokens) {
+  return tokens <= 2 ? GUFO_GEMV_DEPTH : 2;
+}
+__host__ __device__ constexpr int WavesPerSimdFor(int tokens) {
+  return tokens == 1 ? GUFO_GEMV_WAVES_PER_EU : tokens == 2 ? 2 : 1;
+}
+// Row groups per workgroup tile of an expert launch (any column count).
+constexpr uint32_t kMoeGroupsPerTile = kWavesPerGroup * 3;
+
+int g_compute_units = 256;  // set by SetGemvComputeUnits at library init
 
 struct GemvParams {
   GemvLaunch launch;
@@ -174,24 +195,54 @@ __device__ __forceinline__ const float* ColumnX(const Columns<NTOK>& col, uint32
   return p;
 }
 
-// Loads kValues activations; with kSwiGlu the row holds [gate | up] (2*cols values)
-// and the activation is silu(gate) * up, the step between an expert's two products
-// (src/models/qwen35/decoder.cpp:547-549 of the reference).
-template <int kValues, bool kSwiGlu>
-__device__ __forceinline__ void LoadActivations(const float* row, uint32_t at,
-                                                uint32_t cols, float (&v)[kValues]) {
+// The 8 consecutive activations one staging thread handles, as loaded.  With
+// kSwiGlu the row holds [gate | up] (2*cols values) and the activation is
+// silu(gate) * up, the step between an expert's two products
+// (src/models/qwen35/decoder.cpp:547-549 of the reference).  Fetch only issues the
+// loads, so a kernel can have them in flight early; Values waits for them.
+template <bool kSwiGlu>
+struct Octet {
+  float4 lo[2];
+  float4 up[2];
+
+  __device__ __forceinline__ void Fetch(const float* row, uint32_t at, uint32_t cols) {
 #pragma unroll
-  for (int q = 0; q < kValues / 4; ++q) {
-    float4 f = reinterpret_cast<const float4*>(row + at)[q];
-    if (kSwiGlu) {
-      const float4 u = reinterpret_cast<const float4*>(row + cols + at)[q];
-      f = make_float4(Silu(f.x) * u.x, Silu(f.y) * u.y, Silu(f.z) * u.z, Silu(f.w) * u.w);
+    for (int q = 0; q < 2; ++q) {
+      lo[q] = reinterpret_cast<const float4*>(row + at)[q];
+      if (kSwiGlu) up[q] = reinterpret_cast<const float4*>(row + cols + at)[q];
     }
-    v[4 * q + 0] = f.x;
-    v[4 * q + 1] = f.y;
-    v[4 * q + 2] = f.z;
-    v[4 * q + 3] = f.w;
   }
+
+  __device__ __forceinline__ void Values(float (&v)[8]) const {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      float4 f = lo[q];
+      if (kSwiGlu) {
+        const float4 u = up[q];
+        f = make_float4(Silu(f.x) * u.x, Silu(f.y) * u.y, Silu(f.z) * u.z, Silu(f.w) * u.w);
+      }
+      v[4 * q + 0] = f.x;
+      v[4 * q + 1] = f.y;
+      v[4 * q + 2] = f.z;
+      v[4 * q + 3] = f.w;
+    }
+  }
+};
+
+// Which token column and which 8 values of it staging piece `u` is.
+struct OctetIndex {
+  uint32_t token;
+  uint32_t block;
+  uint32_t piece;  // values 8*piece .. +8 of the block
+};
+
+__device__ __forceinline__ OctetIndex IndexOctet(uint32_t u, uint32_t octets_per_token) {
+  OctetIndex ix;
+  ix.token = u / octets_per_token;
+  const uint32_t o = u - ix.token * octets_per_token;
+  ix.block = o >> 5;
+  ix.piece = o & 31;
+  return ix;
 }
 
 // Quantizes all token columns into LDS.  A thread takes 8 consecutive values; the two
@@ -199,21 +250,31 @@ __device__ __forceinline__ void LoadActivations(const float* row, uint32_t at,
 // scale group agree on its largest magnitude and on sum(X) through quad exchanges.
 // The number of 8-value pieces per token is a multiple of 32, so quads are never
 // split by the loop bound.
+// `first` holds the loads of the thread's first piece (u = threadIdx.x), fetched by the
+// caller before it issued its weight loads: memory returns loads in issue order, so
+// this way the wait for x does not also wait for the weights.
 template <int TYPE, int NTOK, bool kSwiGlu>
 __device__ __forceinline__ void StageActivations(const GemvParams& prm,
-                                                 const Columns<NTOK>& col, U32x4* lds) {
+                                                 const Columns<NTOK>& col,
+                                                 const Octet<kSwiGlu>& first, U32x4* lds) {
   constexpr bool kSix = TYPE == kTypeQ6K;
   constexpr uint32_t kSlots = Slots<TYPE>();
   const uint32_t bpp_log2 = prm.bpp_log2;
   const uint32_t positions = 4u << bpp_log2;  // lanes that cover one pass of a row
   const uint32_t octets = prm.launch.blocks_per_row * 32;  // 8-value pieces per token
   for (uint32_t u = threadIdx.x; u < NTOK * octets; u += kThreads) {
-    const uint32_t t = u / octets;
-    const uint32_t o = u - t * octets;
-    const uint32_t block = o >> 5;
-    const uint32_t piece = o & 31;  // values 8*piece .. +8 of the block
+    const OctetIndex ix = IndexOctet(u, octets);
+    const uint32_t t = ix.token;
+    const uint32_t block = ix.block;
+    const uint32_t piece = ix.piece;
     float v[8];
-    LoadActivations<8, kSwiGlu>(ColumnX<NTOK>(col, t), block * 256 + piece * 8, prm.cols, v);
+    if (u == threadIdx.x) {
+      first.Values(v);
+    } else {
+      Octet<kSwiGlu> later;
+      later.Fetch(ColumnX<NTOK>(col, t), block * 256 + piece * 8, prm.cols);
+      later.Values(v);
+    }
     float gmax = 0.0f;
 #pragma unroll
     for (int c = 0; c < 8; ++c) gmax = fmaxf(gmax, fabsf(v[c]));
@@ -471,16 +532,17 @@ __device__ __forceinline__ float GroupTotal(float v, int lanes) {
 
 // One workgroup's share.  Row group g (16 >> bpp_log2 consecutive flat rows) is
 // visited by one wave; this wave takes groups g_first, g_first + g_stride, ... below
-// g_end.  part_shift[p] (optional) is added to part p's row pointer: the byte offset
-// of an expert inside a 3-D tensor.
+// g_end.  part_shift is added to every part's row pointer: the byte offset of an
+// expert inside its 3-D tensor (the parts of one launch share the expert stride).
 template <int TYPE, int NTOK, bool kSwiGlu>
 __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NTOK>& col,
-                                         const size_t* part_shift, uint32_t g_first,
+                                         size_t part_shift, uint32_t g_first,
                                          uint32_t g_stride, uint32_t g_end, U32x4* lds) {
   using Raw = typename RawOf<TYPE>::Type;
   using X = typename XOf<TYPE>::Type;
   constexpr int kBlockBytes = BlockBytes(TYPE);
   constexpr uint32_t kSlots = Slots<TYPE>();
+  constexpr int kDepth = DepthFor(NTOK);  // row visits of weight loads held in registers
 
   const int lane = threadIdx.x & 63;
   const uint32_t bpp_log2 = prm.bpp_log2;
@@ -501,9 +563,8 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
   uint32_t y_index[kDepth];
   bool valid[kDepth];
 
-  const size_t shift0 = part_shift != nullptr ? part_shift[0] : 0;
   const uint8_t* const base0 =
-      prm.launch.part[0].rows + shift0 + static_cast<size_t>(blk_lane) * kBlockBytes;
+      prm.launch.part[0].rows + part_shift + static_cast<size_t>(blk_lane) * kBlockBytes;
   const uint32_t y_offset0 = prm.launch.part[0].y_offset;
   const bool one_part = prm.launch.n_parts == 1;
   auto locate = [&](int d, uint32_t group) {
@@ -515,19 +576,17 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
       return;
     }
     const uint8_t* base = prm.launch.part[0].rows;
-    size_t shift = shift0;
     uint32_t start = 0;
     uint32_t y_offset = y_offset0;
 #pragma unroll
     for (int p = 1; p < kMaxGemvParts; ++p) {
       if (p < static_cast<int>(prm.launch.n_parts) && flat >= prm.start[p]) {
         base = prm.launch.part[p].rows;
-        shift = part_shift != nullptr ? part_shift[p] : 0;
         start = prm.start[p];
         y_offset = prm.launch.part[p].y_offset;
       }
     }
-    row_base[d] = base + shift + static_cast<size_t>(flat - start) * prm.row_bytes +
+    row_base[d] = base + part_shift + static_cast<size_t>(flat - start) * prm.row_bytes +
                   static_cast<size_t>(blk_lane) * kBlockBytes;
     y_index[d] = y_offset + (flat - start);
   };
@@ -537,14 +596,23 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
     }
   };
 
-  // Weight loads first, so that their latency overlaps the staging of x.
+  // The thread's first piece of x, then the first weight loads, then the staging:
+  // both latencies overlap, and the wait for x does not wait for the weights.
+  Octet<kSwiGlu> first_piece;
+  {
+    const uint32_t octets = prm.launch.blocks_per_row * 32;
+    if (threadIdx.x < NTOK * octets) {
+      const OctetIndex ix = IndexOctet(threadIdx.x, octets);
+      first_piece.Fetch(ColumnX<NTOK>(col, ix.token), ix.block * 256 + ix.piece * 8, prm.cols);
+    }
+  }
 #pragma unroll
   for (int d = 0; d < kDepth; ++d) {
     locate(d, g_first + d * g_stride);
     issue(d, 0);
   }
 
-  StageActivations<TYPE, NTOK, kSwiGlu>(prm, col, lds);
+  StageActivations<TYPE, NTOK, kSwiGlu>(prm, col, first_piece, lds);
   __syncthreads();
 
   X x[NTOK];
@@ -594,7 +662,8 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
 // Dense product: token t reads x + t*cols and writes y + t*y_stride; the waves of
 // the whole grid share the row groups round robin.
 template <int TYPE, int NTOK>
-__global__ __launch_bounds__(kThreads) void KquantGemvKernel(
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(NTOK)))) void KquantGemvKernel(
     const GemvParams prm, const float* __restrict__ x, float* __restrict__ y) {
   extern __shared__ __align__(16) U32x4 lds[];
   Columns<NTOK> col;
@@ -604,7 +673,7 @@ __global__ __launch_bounds__(kThreads) void KquantGemvKernel(
     col.y[t] = y + static_cast<size_t>(t) * prm.launch.y_stride;
   }
   const uint32_t wave = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
-  GemvBody<TYPE, NTOK, false>(prm, col, nullptr, wave, gridDim.x * kWavesPerGroup,
+  GemvBody<TYPE, NTOK, false>(prm, col, 0, wave, gridDim.x * kWavesPerGroup,
                               prm.n_groups, lds);
 }
 
@@ -625,30 +694,31 @@ __device__ __forceinline__ void MoeSegmentBody(const GemvParams& prm,
     col.x[t] = moe.x + x_row * moe.x_row_floats;
     col.y[t] = moe.y + static_cast<size_t>(pair) * prm.launch.y_stride;
   }
-  size_t shift[kMaxGemvParts];
-#pragma unroll
-  for (int p = 0; p < kMaxGemvParts; ++p) {
-    shift[p] = static_cast<size_t>(seg.expert) * moe.expert_bytes[p];
-  }
-  const uint32_t groups_per_tile = kWavesPerGroup * kDepth;
-  const uint32_t first = blockIdx.x * groups_per_tile;
-  const uint32_t end = min(first + groups_per_tile, prm.n_groups);
+  const size_t shift = static_cast<size_t>(seg.expert) * moe.expert_bytes;
+  const uint32_t first = blockIdx.x * kMoeGroupsPerTile;
+  const uint32_t end = min(first + kMoeGroupsPerTile, prm.n_groups);
   GemvBody<TYPE, NTOK, kSwiGlu>(prm, col, shift, first + (threadIdx.x >> 6),
                                 kWavesPerGroup, end, lds);
 }
 
-template <int TYPE, bool kSwiGlu>
-__global__ __launch_bounds__(kThreads) void KquantMoeGemvKernel(const GemvParams prm,
-                                                                const MoeGemvArgs moe) {
+// kMaxTok bounds the pairs of a segment (the launch's token count, at most four):
+// a one-token call compiles only the one-column body and keeps its registers.
+template <int TYPE, bool kSwiGlu, int kMaxTok>
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(kMaxTok)))) void KquantMoeGemvKernel(
+    const GemvParams prm, const MoeGemvArgs moe) {
   extern __shared__ __align__(16) U32x4 lds[];
   const uint32_t s = blockIdx.y;
   if (s >= static_cast<uint32_t>(moe.tables->n_segments)) return;
   const MoeSegment seg = moe.segments[s];
-  switch (seg.n_pairs) {
-    case 1: MoeSegmentBody<TYPE, 1, kSwiGlu>(prm, moe, seg, lds); break;
-    case 2: MoeSegmentBody<TYPE, 2, kSwiGlu>(prm, moe, seg, lds); break;
-    case 3: MoeSegmentBody<TYPE, 3, kSwiGlu>(prm, moe, seg, lds); break;
-    default: MoeSegmentBody<TYPE, 4, kSwiGlu>(prm, moe, seg, lds); break;
+  if (kMaxTok == 1 || seg.n_pairs == 1) {
+    MoeSegmentBody<TYPE, 1, kSwiGlu>(prm, moe, seg, lds);
+  } else if (kMaxTok >= 2 && seg.n_pairs == 2) {
+    MoeSegmentBody<TYPE, kMaxTok >= 2 ? 2 : 1, kSwiGlu>(prm, moe, seg, lds);
+  } else if (kMaxTok >= 3 && seg.n_pairs == 3) {
+    MoeSegmentBody<TYPE, kMaxTok >= 3 ? 3 : 1, kSwiGlu>(prm, moe, seg, lds);
+  } else {
+    MoeSegmentBody<TYPE, kMaxTok >= 4 ? 4 : 1, kSwiGlu>(prm, moe, seg, lds);
   }
 }
 
@@ -714,24 +784,33 @@ hipError_t LaunchTyped(const GemvParams& prm, const float* x, int tokens, float*
   }
 }
 
-template <int TYPE>
-hipError_t LaunchMoeTyped(const GemvParams& prm, const MoeGemvArgs& moe, bool swiglu,
-                          dim3 grid, size_t lds_bytes, hipStream_t stream) {
-  if (swiglu) {
-    const hipError_t status = AllowLargeLds(KquantMoeGemvKernel<TYPE, true>, lds_bytes);
-    if (status != hipSuccess) return status;
-    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, true>), grid, dim3(kThreads), lds_bytes,
-                       stream, prm, moe);
-  } else {
-    const hipError_t status = AllowLargeLds(KquantMoeGemvKernel<TYPE, false>, lds_bytes);
-    if (status != hipSuccess) return status;
-    hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, false>), grid, dim3(kThreads), lds_bytes,
-                       stream, prm, moe);
-  }
+template <int TYPE, bool kSwiGlu, int kMaxTok>
+hipError_t LaunchMoeKernel(const GemvParams& prm, const MoeGemvArgs& moe, dim3 grid,
+                           size_t lds_bytes, hipStream_t stream) {
+  const hipError_t status =
+      AllowLargeLds(KquantMoeGemvKernel<TYPE, kSwiGlu, kMaxTok>, lds_bytes);
+  if (status != hipSuccess) return status;
+  hipLaunchKernelGGL((KquantMoeGemvKernel<TYPE, kSwiGlu, kMaxTok>), grid, dim3(kThreads),
+                     lds_bytes, stream, prm, moe);
   return hipGetLastError();
 }
 
+template <int TYPE>
+hipError_t LaunchMoeTyped(const GemvParams& prm, const MoeGemvArgs& moe, bool swiglu,
+                          bool one_token, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+  if (swiglu) {
+    return one_token ? LaunchMoeKernel<TYPE, true, 1>(prm, moe, grid, lds_bytes, stream)
+                     : LaunchMoeKernel<TYPE, true, 4>(prm, moe, grid, lds_bytes, stream);
+  }
+  return one_token ? LaunchMoeKernel<TYPE, false, 1>(prm, moe, grid, lds_bytes, stream)
+                   : LaunchMoeKernel<TYPE, false, 4>(prm, moe, grid, lds_bytes, stream);
+}
+
 }  // namespace
+
+void SetGemvComputeUnits(int compute_units) {
+  if (compute_units > 0) g_compute_units = compute_units;
+}
 
 int GemvMaxTokens(int type, uint32_t blocks_per_row) {
   const size_t per_token = LdsBytes(type, blocks_per_row, 1);
@@ -751,7 +830,10 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
   PlanGemv(type, launch, &prm);
   const size_t lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens);
   uint32_t blocks = (prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
-  if (blocks > kMaxGrid) blocks = kMaxGrid;
+  // Persistent: no more workgroups than are resident at once.
+  const uint32_t resident =
+      static_cast<uint32_t>(g_compute_units) * WavesPerSimdFor(tokens);
+  if (blocks > resident) blocks = resident;
   const dim3 grid(blocks);
   switch (type) {
     case kTypeQ4K: return LaunchTyped<kTypeQ4K>(prm, x, tokens, y, grid, lds_bytes, stream);
@@ -761,22 +843,27 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
 }
 
 hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& moe,
-                         bool swiglu, uint32_t max_segments, hipStream_t stream) {
-  if (!ValidLaunch(type, launch) ||
+                         bool swiglu, uint32_t max_segments, int max_pairs,
+                         hipStream_t stream) {
+  if (!ValidLaunch(type, launch) || max_pairs < 1 ||
       GemvMaxTokens(type, launch.blocks_per_row) < kMaxGemvTokens) {
     return hipErrorInvalidValue;
   }
   if (launch.total_rows == 0 || max_segments == 0) return hipSuccess;
   GemvParams prm;
   PlanGemv(type, launch, &prm);
-  // Sized for the widest segment (four columns); narrower ones use less of it.
-  const size_t lds_bytes = LdsBytes(type, launch.blocks_per_row, kMaxGemvTokens);
-  const uint32_t groups_per_tile = kWavesPerGroup * kDepth;
-  const dim3 grid((prm.n_groups + groups_per_tile - 1) / groups_per_tile, max_segments);
+  // Sized for the widest segment the launch can hold; narrower ones use less of it.
+  const bool one_token = max_pairs == 1;
+  const size_t lds_bytes =
+      LdsBytes(type, launch.blocks_per_row, one_token ? 1 : kMaxGemvTokens);
+  const dim3 grid((prm.n_groups + kMoeGroupsPerTile - 1) / kMoeGroupsPerTile, max_segments);
   switch (type) {
-    case kTypeQ4K: return LaunchMoeTyped<kTypeQ4K>(prm, moe, swiglu, grid, lds_bytes, stream);
-    case kTypeQ5K: return LaunchMoeTyped<kTypeQ5K>(prm, moe, swiglu, grid, lds_bytes, stream);
-    default: return LaunchMoeTyped<kTypeQ6K>(prm, moe, swiglu, grid, lds_bytes, stream);
+    case kTypeQ4K:
+      return LaunchMoeTyped<kTypeQ4K>(prm, moe, swiglu, one_token, grid, lds_bytes, stream);
+    case kTypeQ5K:
+      return LaunchMoeTyped<kTypeQ5K>(prm, moe, swiglu, one_token, grid, lds_bytes, stream);
+    default:
+      return LaunchMoeTyped<kTypeQ6K>(prm, moe, swiglu, one_token, grid, lds_bytes, stream);
   }
 }
 

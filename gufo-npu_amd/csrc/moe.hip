@@ -105,8 +105,9 @@ __global__ __launch_bounds__(64) void RouteKernel(const float* __restrict__ logi
 constexpr int kGroupThreads = 256;
 
 __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
-    const int* __restrict__ ids, int n_pairs, int experts, int* counts, int* offsets,
-    int* pairs, uint8_t* pair_valid, MoeSegment* segments, MoeTables* tables) {
+    const int* __restrict__ ids, int n_pairs, int experts, int capacity, int* counts,
+    int* offsets, int* pairs, uint8_t* pair_valid, MoeSegment* segments,
+    MoeTables* tables) {
   __shared__ int lds_ids[kMaxGroupPairs];
   __shared__ int lds_count[kMaxGroupExperts];
   __shared__ int lds_offset[kMaxGroupExperts + 1];
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
       lds_offset[e] = offset;
       lds_segment0[e] = segment;
       offset += c;
-      segment += (c + kMaxGemvTokens - 1) / kMaxGemvTokens;
+      segment += (c + capacity - 1) / capacity;
       distinct += c != 0 ? 1 : 0;
     }
     lds_offset[experts] = offset;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
       if (lds_ids[i] != e) continue;
       pairs[pos++] = i;
       segments[seg].pair[in_seg++] = i;
-      if (in_seg == kMaxGemvTokens) {
+      if (in_seg == capacity) {
         segments[seg].expert = e;
         segments[seg].n_pairs = in_seg;
         ++seg;
@@ -220,15 +221,15 @@ hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int*
   return hipGetLastError();
 }
 
-hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int* counts,
-                          int* offsets, int* pairs, uint8_t* pair_valid,
+hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int capacity,
+                          int* counts, int* offsets, int* pairs, uint8_t* pair_valid,
                           MoeSegment* segments, MoeTables* tables, hipStream_t stream) {
   if (n_pairs < 0 || n_pairs > kMaxGroupPairs || experts < 1 ||
-      experts > kMaxGroupExperts) {
+      experts > kMaxGroupExperts || capacity < 1 || capacity > kMaxGemvTokens) {
     return hipErrorInvalidValue;
   }
   hipLaunchKernelGGL(MoeGroupKernel, dim3(1), dim3(kGroupThreads), 0, stream, ids,
-                     n_pairs, experts, counts, offsets, pairs, pair_valid, segments,
+                     n_pairs, experts, capacity, counts, offsets, pairs, pair_valid, segments,
                      tables);
   return hipGetLastError();
 }
