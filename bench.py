@@ -25,6 +25,7 @@ import numpy as np
 import __graft_entry__ as entry
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 / bf16
 
 
 def parse_args():
@@ -196,6 +197,22 @@ def run_details(capi, cfg, synth, decode, args):
     for s in sets:
         for m in s:
             m.destroy()
+
+    log("config 5, prefill projection (4096 x 2048 bf16 activations . Q4_K 6144 x 2048):")
+    spec = cfg.CONFIG5
+    mw = capi.Matrix(spec.ggml_type, spec.build(), spec.rows, spec.cols)
+    a_bits = synth.bf16_round(synth.activations(cfg.CONFIG5_TOKENS, spec.cols, cfg.CONFIG5_A_SEED))
+    da = capi.DeviceBuffer.from_array(a_bits)
+    dc = capi.DeviceBuffer(4 * cfg.CONFIG5_TOKENS * spec.rows)
+    ms = time_recorded(capi, [lambda: capi.gemm_q4k_bf16_dev(mw, da, cfg.CONFIG5_TOKENS, dc)] * 4,
+                       reps=10)
+    flops = 2.0 * cfg.CONFIG5_TOKENS * spec.rows * spec.cols
+    log(f"  gemm 4096x6144x2048 (pre-pass + MFMA kernel)  {ms * 1e3:8.2f} us  "
+        f"{flops / ms / 1e9:8.1f} TFLOP/s  {100 * flops / ms / 1e9 / MFMA_PEAK_TFLOPS:5.1f}% of "
+        f"the {MFMA_PEAK_TFLOPS:.0f} TFLOP/s fp16/bf16 peak")
+    mw.destroy()
+    da.free()
+    dc.free()
 
     log("config 4, MoE experts (256 experts, hidden 2048, ffn 512, top-8):")
     gate, up, down = (cfg.CONFIG4[n] for n in ("gate", "up", "down"))

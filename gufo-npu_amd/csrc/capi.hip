@@ -73,6 +73,8 @@ struct State {
   Scratch moe_tables;   // counts, offsets, pairs, valid flags, segments
   Scratch moe_gate_up;  // pairs x 2*ffn
   Scratch moe_out;      // pairs x hidden
+  Scratch gemm_work;    // prefill: fp16 activations + sub-block sums
+  Scratch stage_c;      // prefill, host-pointer variant: device copy of C
 };
 
 State g_state;
@@ -488,6 +490,8 @@ int gufo_hip_shutdown(void) {
   Release(&g_state.moe_tables);
   Release(&g_state.moe_gate_up);
   Release(&g_state.moe_out);
+  Release(&g_state.gemm_work);
+  Release(&g_state.stage_c);
   (void)hipEventDestroy(g_state.timer_begin);
   (void)hipEventDestroy(g_state.timer_end);
   (void)hipStreamDestroy(g_state.stream);
@@ -775,26 +779,52 @@ int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   return CheckMoeIdsLocked();
 }
 
+namespace {
+
+int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* c) {
+  if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
+  if (w->type != GUFO_HIP_Q4_K) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "the prefill GEMM takes Q4_K weights; this matrix has ggml type %d", w->type);
+  }
+  if (m == 0 || w->rows == 0) return GUFO_HIP_OK;
+  if (a == nullptr || c == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a or c is null");
+  if (!Aligned16(a)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a must be 16-byte aligned");
+  const uint32_t nb = static_cast<uint32_t>(w->cols / gufo::kSuperBlock);
+  if (m > (1ull << 24)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens exceed the launch limit", m);
+  }
+  GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmWorkspaceBytes(m, nb)));
+  GUFO_HIP_TRY(gufo::LaunchGemmQ4K(w->data, static_cast<uint32_t>(w->rows), nb, a, m,
+                                   g_state.gemm_work.ptr, c, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
+}  // namespace
+
 int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
                                size_t m, float* c_dev) {
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
-  (void)w;
-  (void)a_bf16_dev;
-  (void)m;
-  (void)c_dev;
-  return Fail(GUFO_HIP_ERR_RUNTIME, "the prefill GEMM is not built into this library yet");
+  return GemmDevLocked(w, a_bf16_dev, m, c_dev);
 }
 
 int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
                            float* c_host) {
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
-  (void)w;
-  (void)a_bf16_host;
-  (void)m;
-  (void)c_host;
-  return Fail(GUFO_HIP_ERR_RUNTIME, "the prefill GEMM is not built into this library yet");
+  if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
+  if (m == 0 || w->rows == 0) return GUFO_HIP_OK;
+  if (a_bf16_host == nullptr || c_host == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a or c is null");
+  }
+  const size_t a_bytes = m * w->cols * sizeof(uint16_t);
+  const size_t c_bytes = m * w->rows * sizeof(float);
+  GUFO_TRY(CopyIn(&g_state.stage_x, a_bf16_host, a_bytes));
+  GUFO_TRY(Reserve(&g_state.stage_c, c_bytes));
+  GUFO_TRY(GemmDevLocked(w, static_cast<const uint16_t*>(g_state.stage_x.ptr), m,
+                         static_cast<float*>(g_state.stage_c.ptr)));
+  return CopyOut(c_host, g_state.stage_c.ptr, c_bytes);
 }
 
 int gufo_hip_capture_begin(void) {

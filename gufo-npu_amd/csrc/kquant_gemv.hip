@@ -60,11 +60,13 @@ constexpr int kBlocksPerPass = 16;  // super-blocks a wave covers per pass (4 la
 #define GUFO_GEMV_WAVES_PER_EU 3
 #endif
 __host__ __device__ constexpr int DepthFor(int tokens) {
-  return tokens <= 2 ? GUFO_GEMV_DEPTH : 2;
+  return tokens <= 2 ? GUFO_GEMV_DEPTH : GUFO_GEMV_DEPTH;
 }
 __host__ __device__ constexpr int WavesPerSimdFor(int tokens) {
-  return tokens == 1 ? GUFO_GEMV_WAVES_PER_EU : tokens == 2 ? 2 : 1;
+  return tokens == 1 ? GUFO_GEMV_WAVES_PER_EU : 2;
 }
+// Up to this many token columns keep their quantized activations in registers.
+constexpr int kResidentColumns = 2;
 // Row groups per workgroup tile of an expert launch (any column count).
 constexpr uint32_t kMoeGroupsPerTile = kWavesPerGroup * 3;
 
@@ -405,8 +407,8 @@ struct RawK4 {
     }
   }
 
-  template <int NTOK>
-  __device__ __forceinline__ void Mac(int lane4, const XK4 (&x)[NTOK],
+  template <int NTOK, typename XSource>
+  __device__ __forceinline__ void Mac(int lane4, const XSource& source,
                                       float (&acc)[NTOK]) const {
     const int p = lane4;
     const float d = HalfBitsToFloat(header.x & 0xFFFFu);
@@ -433,12 +435,13 @@ struct RawK4 {
     }
 #pragma unroll
     for (int t = 0; t < NTOK; ++t) {
-      const float dot_lo = static_cast<float>(CodeDot<8>(lo, x[t].limb[0])) * x[t].xs[0];
-      const float dot_hi = static_cast<float>(CodeDot<8>(hi, x[t].limb[1])) * x[t].xs[1];
+      const XK4 x = source.Get(t);
+      const float dot_lo = static_cast<float>(CodeDot<8>(lo, x.limb[0])) * x.xs[0];
+      const float dot_hi = static_cast<float>(CodeDot<8>(hi, x.limb[1])) * x.xs[1];
       float part = scale0 * dot_lo;
-      part = Fma(-min0, x[t].fx[0], part);
+      part = Fma(-min0, x.fx[0], part);
       part = Fma(scale1, dot_hi, part);
-      part = Fma(-min1, x[t].fx[1], part);
+      part = Fma(-min1, x.fx[1], part);
       acc[t] += part;
     }
   }
@@ -466,8 +469,8 @@ struct RawQ6 {
     d = Load2(blk + 208);
   }
 
-  template <int NTOK>
-  __device__ __forceinline__ void Mac(int lane4, const XQ6 (&x)[NTOK],
+  template <int NTOK, typename XSource>
+  __device__ __forceinline__ void Mac(int lane4, const XSource& source,
                                       float (&acc)[NTOK]) const {
     const int i = lane4 & 1;
     uint32_t codes[4][4];
@@ -488,11 +491,12 @@ struct RawQ6 {
     const float df = HalfBitsToFloat(d);
 #pragma unroll
     for (int t = 0; t < NTOK; ++t) {
+      const XQ6 x = source.Get(t);
       float block = 0.0f;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const int dot = CodeDot<4>(codes[k], x[t].limb[k]) - x[t].sx32[k];
-        block = Fma(scale[k], static_cast<float>(dot) * x[t].xs[k], block);
+        const int dot = CodeDot<4>(codes[k], x.limb[k]) - x.sx32[k];
+        block = Fma(scale[k], static_cast<float>(dot) * x.xs[k], block);
       }
       acc[t] = Fma(df, block, acc[t]);
     }
@@ -506,6 +510,28 @@ struct RawOf {
 template <>
 struct RawOf<kTypeQ6K> {
   using Type = RawQ6;
+};
+
+// Where a visit's arithmetic takes the quantized activations of token column t
+// from: registers (one or two columns: loaded once per pass, reused by every row
+// visit) or LDS (three or four columns would not leave registers for the weight
+// prefetch, so each visit reads them again).
+template <typename X, int NTOK>
+struct ResidentX {
+  X x[NTOK];
+  __device__ __forceinline__ const X& Get(int t) const { return x[t]; }
+};
+
+template <typename X>
+struct LdsX {
+  const U32x4* base;       // this lane's position in column 0 of the current pass
+  uint32_t column_stride;  // 16-byte units between token columns
+  uint32_t positions;
+  __device__ __forceinline__ X Get(int t) const {
+    X x;
+    LoadX(base + static_cast<size_t>(t) * column_stride, positions, &x);
+    return x;
+  }
 };
 
 // ---- cross-lane sum ----------------------------------------------------------------
@@ -615,7 +641,11 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
   StageActivations<TYPE, NTOK, kSwiGlu>(prm, col, first_piece, lds);
   __syncthreads();
 
-  X x[NTOK];
+  constexpr bool kResident = NTOK <= kResidentColumns;
+  ResidentX<X, kResident ? NTOK : 1> resident;
+  LdsX<X> streamed;
+  streamed.column_stride = passes * kSlots * positions;
+  streamed.positions = positions;
   float acc[kDepth][NTOK];
   uint32_t group0 = g_first;  // group of visit 0 of the current iteration
   uint32_t pass = 0;
@@ -627,12 +657,17 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
         for (int t = 0; t < NTOK; ++t) acc[d][t] = 0.0f;
       }
     }
-    if (passes > 1 || group0 == g_first) {
+    const U32x4* pass_base = lds + static_cast<size_t>(pass) * kSlots * positions + position;
+    if (kResident) {
+      if (passes > 1 || group0 == g_first) {
 #pragma unroll
-      for (int t = 0; t < NTOK; ++t) {
-        LoadX(lds + (static_cast<size_t>(t) * passes + pass) * kSlots * positions + position,
-              positions, &x[t]);
+        for (int t = 0; t < (kResident ? NTOK : 1); ++t) {
+          LoadX(pass_base + static_cast<size_t>(t) * streamed.column_stride, positions,
+                &resident.x[t]);
+        }
       }
+    } else {
+      streamed.base = pass_base;
     }
     const bool last_pass = pass + 1 == passes;
     const uint32_t next_pass = last_pass ? 0 : pass + 1;
@@ -641,7 +676,13 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
     for (int d = 0; d < kDepth; ++d) {
       // The arithmetic of this visit, then the loads of the visit that takes over its
       // registers: kDepth - 1 visits stay in flight meanwhile.
-      if (valid[d]) raw[d].Mac(lane4, x, acc[d]);
+      if (valid[d]) {
+        if (kResident) {
+          raw[d].template Mac<NTOK>(lane4, resident, acc[d]);
+        } else {
+          raw[d].template Mac<NTOK>(lane4, streamed, acc[d]);
+        }
+      }
       if (last_pass) {
 #pragma unroll
         for (int t = 0; t < NTOK; ++t) {

@@ -11,88 +11,78 @@ namespace {
 // qwen35::Route (src/models/qwen35/moe.cpp:16-42 of the reference): probabilities
 // exp(logit - max) in double, the k largest in order (the lower index on equal
 // probabilities), weights p/total/top with top = sum of the chosen p/total,
-// floored at the smallest normal fp16.  One wave per token; lane l holds experts
-// l, l+64, ...
+// floored at the smallest normal fp16.
+//
+// One workgroup per token, one thread per expert.  Instead of k rounds of a
+// wave-wide arg-max, every thread counts the experts that precede its own in the
+// reference's order (higher probability, or equal probability and lower index):
+// that count is the expert's slot, and the experts whose count is below k are the
+// chosen ones.  The order is total, so the result does not depend on scheduling.
 
-struct Candidate {
-  double prob;
-  int index;
-};
+constexpr int kRouteThreads = 256;
+constexpr int kRoutePerThread = kMaxRouteExperts / kRouteThreads;
 
-__device__ __forceinline__ Candidate BetterCandidate(Candidate a, Candidate b) {
-  const bool take_b = b.prob > a.prob || (b.prob == a.prob && b.index < a.index);
-  return take_b ? b : a;
-}
-
-constexpr int kRoutePerLane = kMaxRouteExperts / 64;
-
-__global__ __launch_bounds__(64) void RouteKernel(const float* __restrict__ logits,
-                                                  int experts, int k, int* ids,
-                                                  float* weights) {
-  const int lane = threadIdx.x;
+__global__ __launch_bounds__(kRouteThreads) void RouteKernel(
+    const float* __restrict__ logits, int experts, int k, int* ids, float* weights) {
+  __shared__ double lds_prob[kMaxRouteExperts];
+  __shared__ double lds_chosen[kMaxRouteK];
+  __shared__ double lds_wave[kRouteThreads / 64];
+  __shared__ float lds_wave_max[kRouteThreads / 64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
   const float* row = logits + static_cast<size_t>(blockIdx.x) * experts;
 
   float max_logit = -INFINITY;
-  for (int e = lane; e < experts; e += 64) max_logit = fmaxf(max_logit, row[e]);
+  for (int e = tid; e < experts; e += kRouteThreads) max_logit = fmaxf(max_logit, row[e]);
   for (int off = 32; off > 0; off >>= 1) {
     max_logit = fmaxf(max_logit, __shfl_xor(max_logit, off, 64));
   }
+  if (lane == 0) lds_wave_max[wave] = max_logit;
+  __syncthreads();
+  max_logit = fmaxf(fmaxf(lds_wave_max[0], lds_wave_max[1]),
+                    fmaxf(lds_wave_max[2], lds_wave_max[3]));
 
-  // prob < 0 marks "no expert here" or "already chosen".
-  double prob[kRoutePerLane];
+  double prob[kRoutePerThread];
   double total = 0.0;
 #pragma unroll
-  for (int j = 0; j < kRoutePerLane; ++j) {
-    const int e = lane + 64 * j;
-    prob[j] = -1.0;
+  for (int j = 0; j < kRoutePerThread; ++j) {
+    const int e = tid + kRouteThreads * j;
+    prob[j] = 0.0;
     if (e < experts) {
       prob[j] = exp(static_cast<double>(row[e]) - static_cast<double>(max_logit));
+      lds_prob[e] = prob[j];
       total += prob[j];
     }
   }
   for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off, 64);
+  if (lane == 0) lds_wave[wave] = total;
+  __syncthreads();
+  total = (lds_wave[0] + lds_wave[1]) + (lds_wave[2] + lds_wave[3]);
 
-  double my_prob = 0.0;  // lane `slot` keeps the slot's probability
-  int my_index = 0;
-  for (int slot = 0; slot < k; ++slot) {
-    Candidate best;
-    best.prob = -1.0;
-    best.index = 0x7FFFFFFF;
 #pragma unroll
-    for (int j = 0; j < kRoutePerLane; ++j) {
-      Candidate c;
-      c.prob = prob[j];
-      c.index = lane + 64 * j;
-      if (prob[j] >= 0.0) best = BetterCandidate(best, c);
+  for (int j = 0; j < kRoutePerThread; ++j) {
+    const int e = tid + kRouteThreads * j;
+    if (e >= experts) continue;
+    const double mine = prob[j];
+    int before = 0;
+    for (int o = 0; o < experts; ++o) {
+      const double other = lds_prob[o];
+      before += (other > mine || (other == mine && o < e)) ? 1 : 0;
     }
-    for (int off = 32; off > 0; off >>= 1) {
-      Candidate o;
-      o.prob = __shfl_xor(best.prob, off, 64);
-      o.index = __shfl_xor(best.index, off, 64);
-      best = BetterCandidate(best, o);
-    }
-    // The owner retires the winner.
-#pragma unroll
-    for (int j = 0; j < kRoutePerLane; ++j) {
-      if (lane + 64 * j == best.index) prob[j] = -1.0;
-    }
-    if (lane == slot) {
-      my_prob = best.prob;
-      my_index = best.index;
+    if (before < k) {
+      ids[static_cast<size_t>(blockIdx.x) * k + before] = e;
+      lds_chosen[before] = mine;
     }
   }
-
-  // top = sum over slots, in slot order, of p/total.
-  double top = 0.0;
-  for (int slot = 0; slot < k; ++slot) {
-    const double p = __shfl(my_prob, slot, 64);
-    top += p / total;
-  }
-  top = fmax(top, 6.103515625e-5);
-  if (lane < k) {
-    ids[static_cast<size_t>(blockIdx.x) * k + lane] = my_index;
-    weights[static_cast<size_t>(blockIdx.x) * k + lane] =
-        static_cast<float>(my_prob / total / top);
+  __syncthreads();
+  if (tid < k) {
+    // top = sum over slots, in slot order, of p/total.
+    double top = 0.0;
+    for (int slot = 0; slot < k; ++slot) top += lds_chosen[slot] / total;
+    top = fmax(top, 6.103515625e-5);
+    weights[static_cast<size_t>(blockIdx.x) * k + tid] =
+        static_cast<float>(lds_chosen[tid] / total / top);
   }
 }
 
@@ -103,6 +93,30 @@ __global__ __launch_bounds__(64) void RouteKernel(const float* __restrict__ logi
 // ascending without atomics on positions.
 
 constexpr int kGroupThreads = 256;
+constexpr int kGroupPerThread = kMaxGroupExperts / kGroupThreads;
+
+// Exclusive prefix sums over the workgroup of one value per thread; *total gets the
+// sum.  `scratch` holds one int per wave.
+__device__ __forceinline__ int BlockExclusiveScan(int value, int* scratch, int* total) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  int inclusive = value;
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(inclusive, off, 64);
+    if (lane >= off) inclusive += up;
+  }
+  __syncthreads();  // scratch may still be read by an earlier scan
+  if (lane == 63) scratch[wave] = inclusive;
+  __syncthreads();
+  int before = 0;
+  int sum = 0;
+  for (int w = 0; w < kGroupThreads / 64; ++w) {
+    if (w < wave) before += scratch[w];
+    sum += scratch[w];
+  }
+  *total = sum;
+  return before + inclusive - value;
+}
 
 __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
     const int* __restrict__ ids, int n_pairs, int experts, int capacity, int* counts,
@@ -110,13 +124,12 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
     MoeTables* tables) {
   __shared__ int lds_ids[kMaxGroupPairs];
   __shared__ int lds_count[kMaxGroupExperts];
-  __shared__ int lds_offset[kMaxGroupExperts + 1];
-  __shared__ int lds_segment0[kMaxGroupExperts + 1];
+  __shared__ int lds_scan[kGroupThreads / 64];
   __shared__ int lds_invalid;
   const int tid = threadIdx.x;
 
   if (tid == 0) lds_invalid = 0;
-  for (int e = tid; e < experts; e += kGroupThreads) lds_count[e] = 0;
+  for (int e = tid; e < kMaxGroupExperts; e += kGroupThreads) lds_count[e] = 0;
   __syncthreads();
   for (int i = tid; i < n_pairs; i += kGroupThreads) {
     const int e = ids[i];
@@ -130,42 +143,48 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
     }
   }
   __syncthreads();
+
+  // Thread t owns experts t*kGroupPerThread .. +kGroupPerThread: their pair counts,
+  // segment counts and "chosen at all" flags, scanned across the workgroup.
+  int count[kGroupPerThread];
+  int my_pairs = 0;
+  int my_segments = 0;
+  int my_distinct = 0;
+#pragma unroll
+  for (int j = 0; j < kGroupPerThread; ++j) {
+    count[j] = lds_count[tid * kGroupPerThread + j];
+    my_pairs += count[j];
+    my_segments += (count[j] + capacity - 1) / capacity;
+    my_distinct += count[j] != 0 ? 1 : 0;
+  }
+  int total_pairs, total_segments, total_distinct;
+  int pair_offset = BlockExclusiveScan(my_pairs, lds_scan, &total_pairs);
+  int segment_offset = BlockExclusiveScan(my_segments, lds_scan, &total_segments);
+  BlockExclusiveScan(my_distinct, lds_scan, &total_distinct);
   if (tid == 0) {
-    int offset = 0;
-    int segment = 0;
-    int distinct = 0;
-    for (int e = 0; e < experts; ++e) {
-      const int c = lds_count[e];
-      lds_offset[e] = offset;
-      lds_segment0[e] = segment;
-      offset += c;
-      segment += (c + capacity - 1) / capacity;
-      distinct += c != 0 ? 1 : 0;
-    }
-    lds_offset[experts] = offset;
-    lds_segment0[experts] = segment;
-    tables->n_segments = segment;
-    tables->n_distinct = distinct;
+    tables->n_segments = total_segments;
+    tables->n_distinct = total_distinct;
     tables->n_invalid = lds_invalid;
     tables->pad = 0;
-  }
-  __syncthreads();
-  for (int e = tid; e <= experts; e += kGroupThreads) {
-    offsets[e] = lds_offset[e];
-    if (e < experts) counts[e] = lds_count[e];
-  }
-  // Invalid pairs go last so that `pairs` stays a permutation of the pair ids.
-  if (tid == 0) {
-    int pos = lds_offset[experts];
-    for (int i = 0; i < n_pairs; ++i) {
+    offsets[experts] = total_pairs;
+    // Invalid pairs go last so that `pairs` stays a permutation of the pair ids.
+    int pos = total_pairs;
+    for (int i = 0; i < n_pairs && pos < n_pairs; ++i) {
       if (lds_ids[i] < 0) pairs[pos++] = i;
     }
   }
-  for (int e = tid; e < experts; e += kGroupThreads) {
-    const int c = lds_count[e];
+#pragma unroll
+  for (int j = 0; j < kGroupPerThread; ++j) {
+    const int e = tid * kGroupPerThread + j;
+    if (e >= experts) break;
+    const int c = count[j];
+    counts[e] = c;
+    offsets[e] = pair_offset;
+    int pos = pair_offset;
+    int seg = segment_offset;
+    pair_offset += c;
+    segment_offset += (c + capacity - 1) / capacity;
     if (c == 0) continue;
-    int pos = lds_offset[e];
-    int seg = lds_segment0[e];
     int in_seg = 0;
     for (int i = 0; i < n_pairs; ++i) {
       if (lds_ids[i] != e) continue;
@@ -174,6 +193,7 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
       if (in_seg == capacity) {
         segments[seg].expert = e;
         segments[seg].n_pairs = in_seg;
+        for (int f = in_seg; f < kMaxGemvTokens; ++f) segments[seg].pair[f] = i;
         ++seg;
         in_seg = 0;
       }
@@ -181,8 +201,8 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
     if (in_seg != 0) {
       segments[seg].expert = e;
       segments[seg].n_pairs = in_seg;
-      for (int j = in_seg; j < kMaxGemvTokens; ++j) {
-        segments[seg].pair[j] = segments[seg].pair[0];
+      for (int f = in_seg; f < kMaxGemvTokens; ++f) {
+        segments[seg].pair[f] = segments[seg].pair[0];
       }
     }
   }
@@ -216,8 +236,8 @@ hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int*
     return hipErrorInvalidValue;
   }
   if (tokens == 0) return hipSuccess;
-  hipLaunchKernelGGL(RouteKernel, dim3(tokens), dim3(64), 0, stream, logits, experts, k,
-                     ids, weights);
+  hipLaunchKernelGGL(RouteKernel, dim3(tokens), dim3(kRouteThreads), 0, stream, logits,
+                     experts, k, ids, weights);
   return hipGetLastError();
 }
 
@@ -229,8 +249,8 @@ hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int capacity
     return hipErrorInvalidValue;
   }
   hipLaunchKernelGGL(MoeGroupKernel, dim3(1), dim3(kGroupThreads), 0, stream, ids,
-                     n_pairs, experts, capacity, counts, offsets, pairs, pair_valid, segments,
-                     tables);
+                     n_pairs, experts, capacity, counts, offsets, pairs, pair_valid,
+                     segments, tables);
   return hipGetLastError();
 }
 

@@ -1,0 +1,86 @@
+"""Parity of the prefill GEMM (Q4_K weights x bf16 activations on the matrix cores)
+with the CPU checker and the golden reference slice, through the C-ABI.
+
+Bar: rel-L2 <= 1e-3 against dequantize + double sum over the same bf16 activation
+values (the bar stated for this kernel); in practice the kernel is ~1e-6."""
+import numpy as np
+import pytest
+
+from conftest import GOLDEN
+from gufo_npu_amd import configs as cfg
+from gufo_npu_amd import synth
+
+pytestmark = pytest.mark.gpu
+TOLERANCE = 1e-3
+
+
+def say(*args):
+    print(*args, flush=True)
+
+
+def bf16_activations(tokens, cols, seed):
+    bits = synth.bf16_round(synth.activations(tokens, cols, seed))
+    return bits, synth.bf16_to_float(bits)
+
+
+@pytest.mark.parametrize("tokens,rows,cols", [(128, 128, 256), (1, 32, 512), (77, 200, 512),
+                                              (300, 129, 2048), (130, 257, 768)])
+def test_gemm_parity_small_and_ragged(hip, oracle, tokens, rows, cols):
+    say("gemm", tokens, rows, cols)
+    seed = 7000 + tokens + rows + cols
+    w = synth.kquant_matrix(synth.Q4_K, rows, cols, seed)
+    bits, a = bf16_activations(tokens, cols, seed + 1)
+    m = hip.Matrix(synth.Q4_K, w, rows, cols)
+    got = hip.gemm_q4k_bf16(m, bits)
+    want = oracle.matmul([(synth.Q4_K, w, 0, rows)], a, precision="double", threads=8)
+    assert got.shape == want.shape == (tokens, rows)
+    assert oracle.rel_l2(got, want) <= TOLERANCE
+    # every row of C is the matrix-vector product of that token
+    for t in sorted({0, tokens // 2, tokens - 1}):
+        single = hip.gemv([hip.whole(m)], a[t:t + 1], 1)
+        assert oracle.rel_l2(got[t], single[0]) <= 1e-4
+    m.destroy()
+
+
+def test_gemm_unit_activations_return_the_weights(hip, oracle):
+    # a = unit vectors (exact in bf16): C[t] is column t of the dequantized matrix.
+    say("gemm identity")
+    rows, cols = 64, 512
+    w = synth.kquant_matrix(synth.Q4_K, rows, cols, 99)
+    m = hip.Matrix(synth.Q4_K, w, rows, cols)
+    bits = synth.bf16_round(np.eye(cols, dtype=np.float32))
+    got = hip.gemm_q4k_bf16(m, bits)
+    want = np.stack([oracle.dequantize(synth.Q4_K, w[r], cols) for r in range(rows)], axis=1)
+    assert oracle.rel_l2(got, want) <= 1e-6
+    m.destroy()
+
+
+def test_gemm_rejects_other_types(hip):
+    say("gemm type check")
+    w = synth.kquant_matrix(synth.Q6_K, 32, 256, 1)
+    m = hip.Matrix(synth.Q6_K, w, 32, 256)
+    with pytest.raises(hip.InvalidArgumentError):
+        hip.gemm_q4k_bf16(m, np.zeros((4, 256), np.uint16))
+    m.destroy()
+
+
+def test_config5_prefill_projection(hip, oracle):
+    # Config 5: activations 4096 x 2048 bf16 times Q4_K 6144 x 2048.
+    say("config 5")
+    spec = cfg.CONFIG5
+    w = spec.build()
+    bits, a = bf16_activations(cfg.CONFIG5_TOKENS, spec.cols, cfg.CONFIG5_A_SEED)
+    m = hip.Matrix(spec.ggml_type, w, spec.rows, spec.cols)
+    got = hip.gemm_q4k_bf16(m, bits)
+    golden = np.load(GOLDEN / "config5_prefill_slice.npz")
+    tokens = golden["tokens"]
+    assert oracle.rel_l2(got[tokens][:, ::8], golden["c_double_every8"]) <= TOLERANCE
+    # other token rows against the CPU checker, and against the GEMV kernel
+    pick = np.array([1, 777, 2049, 4095])
+    want = oracle.matmul([(spec.ggml_type, w, 0, spec.rows)], a[pick], precision="double",
+                         threads=8)
+    assert oracle.rel_l2(got[pick], want) <= TOLERANCE
+    single = hip.gemv([hip.whole(m)], a[pick], len(pick))
+    assert oracle.rel_l2(got[pick], single) <= 1e-4
+    say("config 5 rel-L2 vs double", oracle.rel_l2(got[pick], want))
+    m.destroy()
