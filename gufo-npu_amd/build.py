@@ -40,17 +40,18 @@ def build_library() -> Path:
 
 
 def build_host_tests() -> list[Path]:
-    """The C++ adapter's own test program (plain main(), like the reference's tests)."""
-    built = []
+    """The C++ adapter's own test program (plain main(), like the reference's tests).
+    It links the library and, as its checker, the CPU restatement in oracle/."""
     source = HOST / "hip_projections_test.cpp"
-    if source.exists():
-        target = LIB_DIR / "hip_projections_test"
-        _run(["g++", "-std=c++20", "-O2", "-Wall", "-Wextra", "-I", str(ROOT / "include"),
-              "-I", str(HOST), "-o", str(target), str(source),
-              str(HOST / "hip_projections.cpp"), "-L", str(LIB_DIR), "-lgufo_hip",
-              "-Wl,-rpath,$ORIGIN", "-pthread"])
-        built.append(target)
-    return built
+    oracle_dir = ROOT / "oracle"
+    subprocess.run(["make", "-s", "-C", str(oracle_dir), "all"], check=True)
+    target = LIB_DIR / "hip_projections_test"
+    _run(["g++", "-std=c++20", "-O2", "-mf16c", "-Wall", "-Wextra", "-I", str(ROOT / "include"),
+          "-I", str(HOST), "-I", str(oracle_dir), "-o", str(target), str(source),
+          str(HOST / "hip_projections.cpp"), "-L", str(LIB_DIR), "-lgufo_hip",
+          "-L", str(oracle_dir), "-lkquant_oracle",
+          "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/../../oracle", "-pthread"])
+    return [target]
 
 
 def build_all() -> None:

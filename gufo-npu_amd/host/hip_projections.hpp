@@ -1,0 +1,138 @@
+// C++ host side of the MI355X backend: the reference's operator interface for the
+// matrix products of a Qwen3.5 / Qwen3.6 forward pass, served by the C-ABI library
+// (include/gufo_hip.h).
+//
+// `Stage` and `Projections` repeat qwen35::Stage and qwen35::Projections
+// (src/models/qwen35/projections.hpp:14-59 of the reference) name for name, so a
+// consumer that holds a `const Projections&` (Decoder, Reference, the test
+// decorators) can be handed a HipProjections.  HipProjections takes the place of
+// GgufProjections (src/models/qwen35/gguf_projections.hpp:19-58): same methods, same
+// output layout (each row one token, the stage's matrices concatenated), same
+// exceptions.  Where GgufProjections reads its tensors out of a mapped GGUF file,
+// this class is handed them as `Tensor` records - the GGUF reader itself is not part
+// of this backend - and copies them to HBM once.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+struct gufo_hip_matrix;
+
+namespace gufo_hip {
+
+// qwen35::Stage (projections.hpp:14-39): the products grouped by shared input.
+enum class Stage {
+  kLinearIn,     // [qkv | z | alpha | beta]
+  kAttentionIn,  // [q and gate | k | v]
+  kMixerOut,     // ssm_out or attn_output: hidden
+  kFfnIn,        // [gate | up]: the dense FFN or the MoE shared expert
+  kFfnDown,      // ffn_down: hidden
+  kLmHead,       // vocab
+  kRouter,       // [expert logits | shared-expert gate logit]
+  kExpertIn,     // a routed expert's [gate | up]; ApplyExpert only
+  kExpertDown,   // a routed expert's down projection; ApplyExpert only
+  kMtpIn,        // nextn.eh_proj
+};
+
+// qwen35::Projections (projections.hpp:45-59).
+class Projections {
+public:
+  virtual ~Projections() = default;
+  // y[t] = W x[t] for `tokens` rows of the stage's input width; writes `tokens` rows of
+  // the stage's output width.
+  virtual void Apply(Stage stage, int layer, const float* x, int tokens, float* y) const = 0;
+  // The same for routed expert `expert` of an MoE layer (kExpertIn or kExpertDown).
+  virtual void ApplyExpert(Stage /*stage*/, int /*layer*/, int /*expert*/, const float* /*x*/,
+                           int /*tokens*/, float* /*y*/) const {
+    throw std::logic_error("qwen35: these projections have no MoE experts");
+  }
+};
+
+// A weight tensor as a GGUF file describes it (gguf::TensorInfo,
+// src/core/gguf.hpp:40-54): ggml order, shape[0] is the contiguous (row) dimension, so
+// a matrix is [cols, rows] and an expert tensor [cols, rows, experts].  `data` points
+// at the blocks as stored; it is read during construction only.
+struct Tensor {
+  std::string name;
+  int ggml_type = 0;  // 12 = Q4_K, 13 = Q5_K, 14 = Q6_K
+  std::vector<std::uint64_t> shape;
+  const std::uint8_t* data = nullptr;
+};
+
+// The tensors of one layer by stage, as GgufProjections::Layer groups them
+// (gguf_projections.cpp:80-91).  A stage a layer does not have stays empty.
+struct LayerTensors {
+  std::vector<Tensor> linear_in;
+  std::vector<Tensor> attention_in;
+  std::vector<Tensor> mixer_out;
+  std::vector<Tensor> ffn_in;
+  std::vector<Tensor> ffn_down;
+  std::vector<Tensor> router;
+  std::vector<Tensor> mtp_in;
+  // MoE layers: ffn_gate_exps, ffn_up_exps [hidden, expert_ffn, experts] and
+  // ffn_down_exps [expert_ffn, hidden, experts].  Leave `data` null for a dense layer.
+  Tensor gate_exps;
+  Tensor up_exps;
+  Tensor down_exps;
+};
+
+struct ModelTensors {
+  int hidden = 0;
+  int experts = 0;     // 0 for a dense model
+  int expert_ffn = 0;
+  Tensor lm_head;      // [hidden, vocab]
+  std::vector<LayerTensors> layers;
+};
+
+class HipProjections : public Projections {
+public:
+  // Initialises the library on `device`, checks every tensor's shape and uploads the
+  // weights.  Throws std::runtime_error when no MI355X is available (as the
+  // reference's NPU stub does, src/npu/gemv_stub.cpp:8-10) or a shape is wrong
+  // (gguf_projections.cpp:27-46), std::invalid_argument for a row that is not a whole
+  // number of blocks or a type this backend does not take (src/core/quant.cpp:199,224).
+  explicit HipProjections(const ModelTensors& model, int device = 0);
+  ~HipProjections() override;
+  HipProjections(const HipProjections&) = delete;
+  HipProjections& operator=(const HipProjections&) = delete;
+
+  void Apply(Stage stage, int layer, const float* x, int tokens, float* y) const override;
+  void ApplyExpert(Stage stage, int layer, int expert, const float* x, int tokens,
+                   float* y) const override;
+
+  // Input and output widths of a stage (StageInputs / StageOutputs,
+  // src/models/qwen35/reference.cpp:609-648), from the uploaded tensors.
+  std::size_t StageInputs(Stage stage, int layer) const;
+  std::size_t StageOutputs(Stage stage, int layer) const;
+
+  // qwen35::Route (src/models/qwen35/moe.cpp:16-42) on the device.
+  void Route(const float* logits, int tokens, int k, int* chosen, float* weights) const;
+  // The routed experts of one MoE layer in one call: what Decoder::MoeFfn /
+  // Reference::Ffn compute with a Route and 2 k ApplyExpert calls
+  // (src/models/qwen35/decoder.cpp:530-558, reference.cpp:562-606), without the
+  // shared expert.  Tokens are grouped by expert on the device.
+  void RoutedFfn(int layer, const float* x, int tokens, const int* chosen, const float* weights,
+                 int k, float* y) const;
+
+private:
+  struct Matrix {
+    gufo_hip_matrix* handle = nullptr;
+    std::size_t rows = 0;
+    std::size_t cols = 0;
+  };
+  struct Layer;
+  const std::vector<Matrix>* StageMatrices(Stage stage, int layer) const;
+  Matrix Upload(const Tensor& tensor, std::uint64_t experts);
+  void Release() noexcept;
+
+  int hidden_ = 0;
+  int experts_ = 0;
+  int expert_ffn_ = 0;
+  std::vector<Matrix> lm_head_;
+  std::vector<Layer> layers_;
+};
+
+}  // namespace gufo_hip

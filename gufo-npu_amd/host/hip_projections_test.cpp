@@ -1,0 +1,359 @@
+// HipProjections against the CPU checker, in the style of the reference's own tests
+// (plain main(), one line per case, exit 1 on failure): every stage of a dense and of
+// an MoE layer through Apply / ApplyExpert, the layout of concatenated outputs, the
+// routed-expert call, a decorator over the interface, and the exceptions.
+//
+//   hip_projections_test                  needs an MI355X
+//   hip_projections_test --no-device      on a machine without one: the constructor
+//                                         must throw std::runtime_error
+//
+// The checker is oracle/kquant_oracle.c (dequantize + double sum), linked in; the
+// bar is rel-L2 <= 1e-4 as for the kernels.
+#include <immintrin.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "hip_projections.hpp"
+#include "kquant_oracle.h"
+
+namespace {
+
+using gufo_hip::HipProjections;
+using gufo_hip::LayerTensors;
+using gufo_hip::ModelTensors;
+using gufo_hip::Stage;
+using gufo_hip::Tensor;
+
+constexpr double kTolerance = 1e-4;
+int g_failures = 0;
+
+void Report(const std::string& name, bool ok, double value = -1) {
+  if (value >= 0) {
+    std::printf("%s: %.2e %s\n", name.c_str(), value, ok ? "ok" : "FAIL");
+  } else {
+    std::printf("%s %s\n", name.c_str(), ok ? "ok" : "FAIL");
+  }
+  std::fflush(stdout);
+  g_failures += ok ? 0 : 1;
+}
+
+// Random blocks with finite fp16 scales (|N(0, 0.02)|), as the bench generates them.
+struct Weights {
+  int type;
+  std::size_t rows, cols;
+  std::vector<std::uint8_t> bytes;
+};
+
+std::uint16_t ToHalf(float f) {
+  return static_cast<std::uint16_t>(_cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT));
+}
+
+Weights RandomWeights(int type, std::size_t rows, std::size_t cols, std::mt19937& rng) {
+  Weights w{type, rows, cols, {}};
+  const std::size_t block = gufo_oracle_block_bytes(type);
+  w.bytes.resize(rows * cols / 256 * block);
+  for (auto& b : w.bytes) b = static_cast<std::uint8_t>(rng());
+  std::normal_distribution<float> normal(0.0f, 0.02f);
+  for (std::size_t at = 0; at < w.bytes.size(); at += block) {
+    if (type == GUFO_ORACLE_Q6_K) {
+      const std::uint16_t d = ToHalf(std::fabs(normal(rng)));
+      std::memcpy(&w.bytes[at + 208], &d, 2);
+    } else {
+      const std::uint16_t d = ToHalf(std::fabs(normal(rng)));
+      const std::uint16_t dmin = ToHalf(std::fabs(normal(rng)));
+      std::memcpy(&w.bytes[at], &d, 2);
+      std::memcpy(&w.bytes[at + 2], &dmin, 2);
+    }
+  }
+  return w;
+}
+
+Tensor AsTensor(const std::string& name, const Weights& w, std::uint64_t experts = 0) {
+  Tensor t;
+  t.name = name;
+  t.ggml_type = w.type;
+  t.data = w.bytes.data();
+  if (experts != 0) {
+    t.shape = {w.cols, w.rows / experts, experts};
+  } else {
+    t.shape = {w.cols, w.rows};
+  }
+  return t;
+}
+
+std::vector<float> RandomActivations(std::size_t n, std::mt19937& rng, float scale = 1.0f) {
+  std::normal_distribution<float> normal(0.0f, 1.0f);
+  std::vector<float> x(n);
+  for (auto& v : x) v = scale * normal(rng);
+  return x;
+}
+
+double RelL2(const std::vector<float>& got, const std::vector<float>& want) {
+  double num = 0, den = 0;
+  for (std::size_t i = 0; i < want.size(); ++i) {
+    const double d = static_cast<double>(got[i]) - want[i];
+    num += d * d;
+    den += static_cast<double>(want[i]) * want[i];
+  }
+  return std::sqrt(num / (den > 0 ? den : 1));
+}
+
+// y = [W_0 x | W_1 x | ...] by the checker, double accumulation.
+std::vector<float> Expected(const std::vector<const Weights*>& parts,
+                            const std::vector<std::size_t>& first,
+                            const std::vector<std::size_t>& rows, const std::vector<float>& x,
+                            int tokens) {
+  std::vector<const std::uint8_t*> data;
+  std::vector<int> types;
+  std::size_t stride = 0;
+  for (std::size_t p = 0; p < parts.size(); ++p) {
+    data.push_back(parts[p]->bytes.data());
+    types.push_back(parts[p]->type);
+    stride += rows[p];
+  }
+  std::vector<float> y(static_cast<std::size_t>(tokens) * stride);
+  gufo_oracle_matmul(static_cast<int>(parts.size()), data.data(), types.data(), first.data(),
+                     rows.data(), parts[0]->cols, x.data(), tokens, y.data(), 1, 4);
+  return y;
+}
+
+std::vector<float> ExpectedWhole(const std::vector<const Weights*>& parts,
+                                 const std::vector<float>& x, int tokens) {
+  std::vector<std::size_t> first(parts.size(), 0), rows;
+  for (const Weights* w : parts) rows.push_back(w->rows);
+  return Expected(parts, first, rows, x, tokens);
+}
+
+template <typename Exception, typename Fn>
+bool Throws(Fn&& fn) {
+  try {
+    fn();
+  } catch (const Exception&) {
+    return true;
+  } catch (...) {
+    return false;
+  }
+  return false;
+}
+
+// A decorator over the interface, as the reference's tests wrap their projections
+// (RoutingLog, FollowRouting): counts the calls and forwards them.
+class Counting : public gufo_hip::Projections {
+public:
+  explicit Counting(const gufo_hip::Projections& inner) : inner_(inner) {}
+  void Apply(Stage stage, int layer, const float* x, int tokens, float* y) const override {
+    ++calls;
+    inner_.Apply(stage, layer, x, tokens, y);
+  }
+  void ApplyExpert(Stage stage, int layer, int expert, const float* x, int tokens,
+                   float* y) const override {
+    ++calls;
+    inner_.ApplyExpert(stage, layer, expert, x, tokens, y);
+  }
+  mutable int calls = 0;
+
+private:
+  const gufo_hip::Projections& inner_;
+};
+
+int RunNoDevice() {
+  std::mt19937 rng(1);
+  const Weights head = RandomWeights(GUFO_ORACLE_Q4_K, 64, 256, rng);
+  ModelTensors model;
+  model.hidden = 256;
+  model.lm_head = AsTensor("token_embd.weight", head);
+  Report("constructor without a device throws std::runtime_error",
+         Throws<std::runtime_error>([&] { HipProjections p(model); }));
+  return g_failures == 0 ? 0 : 1;
+}
+
+void RunDense(std::mt19937& rng) {
+  const std::size_t hidden = 512, ffn = 768, vocab = 1000, attn = 256, kv = 128;
+  const Weights q = RandomWeights(GUFO_ORACLE_Q5_K, 2 * attn, hidden, rng);
+  const Weights k = RandomWeights(GUFO_ORACLE_Q5_K, kv, hidden, rng);
+  const Weights v = RandomWeights(GUFO_ORACLE_Q6_K, kv, hidden, rng);
+  const Weights o = RandomWeights(GUFO_ORACLE_Q4_K, hidden, attn, rng);
+  const Weights gate = RandomWeights(GUFO_ORACLE_Q4_K, ffn, hidden, rng);
+  const Weights up = RandomWeights(GUFO_ORACLE_Q4_K, ffn, hidden, rng);
+  const Weights down = RandomWeights(GUFO_ORACLE_Q6_K, hidden, ffn, rng);
+  const Weights head = RandomWeights(GUFO_ORACLE_Q6_K, vocab, hidden, rng);
+
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  model.lm_head = AsTensor("token_embd.weight", head);
+  LayerTensors layer;
+  layer.attention_in = {AsTensor("blk.0.attn_q.weight", q), AsTensor("blk.0.attn_k.weight", k),
+                        AsTensor("blk.0.attn_v.weight", v)};
+  layer.mixer_out = {AsTensor("blk.0.attn_output.weight", o)};
+  layer.ffn_in = {AsTensor("blk.0.ffn_gate.weight", gate), AsTensor("blk.0.ffn_up.weight", up)};
+  layer.ffn_down = {AsTensor("blk.0.ffn_down.weight", down)};
+  model.layers.push_back(layer);
+  const HipProjections proj(model);
+  const Counting counted(proj);
+
+  struct Case {
+    const char* name;
+    Stage stage;
+    int layer;
+    std::vector<const Weights*> parts;
+  };
+  const Case cases[] = {
+      {"kAttentionIn [q|k|v] Q5_K,Q5_K,Q6_K", Stage::kAttentionIn, 0, {&q, &k, &v}},
+      {"kMixerOut Q4_K", Stage::kMixerOut, 0, {&o}},
+      {"kFfnIn [gate|up] Q4_K", Stage::kFfnIn, 0, {&gate, &up}},
+      {"kFfnDown Q6_K", Stage::kFfnDown, 0, {&down}},
+      {"kLmHead Q6_K", Stage::kLmHead, -1, {&head}},
+  };
+  for (const Case& c : cases) {
+    for (const int tokens : {1, 3, 5}) {
+      const std::size_t in = c.parts[0]->cols;
+      const auto x = RandomActivations(static_cast<std::size_t>(tokens) * in, rng);
+      const auto want = ExpectedWhole(c.parts, x, tokens);
+      std::vector<float> got(want.size(), -7.0f);
+      counted.Apply(c.stage, c.layer, x.data(), tokens, got.data());
+      const double err = RelL2(got, want);
+      Report(std::string(c.name) + " tokens=" + std::to_string(tokens), err <= kTolerance, err);
+      if (proj.StageInputs(c.stage, c.layer) != in ||
+          proj.StageOutputs(c.stage, c.layer) * tokens != want.size()) {
+        Report(std::string(c.name) + " stage widths", false);
+      }
+    }
+  }
+  Report("decorator forwarded every call", counted.calls == 15);
+
+  // tokens = 0 writes nothing; a stage this layer does not have throws.
+  float untouched = 3.0f;
+  proj.Apply(Stage::kFfnIn, 0, nullptr, 0, &untouched);
+  Report("tokens = 0 is a no-op", untouched == 3.0f);
+  const auto x = RandomActivations(hidden, rng);
+  std::vector<float> y(4096);
+  Report("missing stage throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.Apply(Stage::kRouter, 0, x.data(), 1, y.data());
+         }));
+  Report("expert stage through Apply throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.Apply(Stage::kExpertIn, 0, x.data(), 1, y.data());
+         }));
+  Report("ApplyExpert on a dense model throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.ApplyExpert(Stage::kExpertIn, 0, 0, x.data(), 1, y.data());
+         }));
+  Report("layer out of range throws std::out_of_range", Throws<std::out_of_range>([&] {
+           proj.Apply(Stage::kFfnIn, 3, x.data(), 1, y.data());
+         }));
+  Report("negative token count throws std::invalid_argument", Throws<std::invalid_argument>([&] {
+           proj.Apply(Stage::kFfnIn, 0, x.data(), -1, y.data());
+         }));
+
+  // Construction checks.
+  ModelTensors bad = model;
+  bad.layers[0].ffn_in[1].shape = {256, ffn};  // up does not share gate's input
+  const Weights narrow = RandomWeights(GUFO_ORACLE_Q4_K, ffn, 256, rng);
+  bad.layers[0].ffn_in[1].data = narrow.bytes.data();
+  Report("mismatched stage input throws std::runtime_error",
+         Throws<std::runtime_error>([&] { HipProjections p(bad); }));
+  bad = model;
+  bad.layers[0].ffn_down[0].shape = {ffn, hidden, 2};
+  Report("wrong rank throws std::runtime_error",
+         Throws<std::runtime_error>([&] { HipProjections p(bad); }));
+  bad = model;
+  bad.layers[0].ffn_down[0].shape = {700, hidden};
+  Report("partial block throws std::invalid_argument",
+         Throws<std::invalid_argument>([&] { HipProjections p(bad); }));
+  bad = model;
+  bad.layers[0].ffn_down[0].ggml_type = 8;
+  Report("unsupported type throws std::invalid_argument",
+         Throws<std::invalid_argument>([&] { HipProjections p(bad); }));
+}
+
+void RunMoe(std::mt19937& rng) {
+  const int experts = 8, top = 3;
+  const std::size_t hidden = 512, ffn = 256;
+  const Weights gate = RandomWeights(GUFO_ORACLE_Q4_K, experts * ffn, hidden, rng);
+  const Weights up = RandomWeights(GUFO_ORACLE_Q4_K, experts * ffn, hidden, rng);
+  const Weights down = RandomWeights(GUFO_ORACLE_Q5_K, experts * hidden, ffn, rng);
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  model.experts = experts;
+  model.expert_ffn = static_cast<int>(ffn);
+  LayerTensors layer;
+  layer.gate_exps = AsTensor("blk.0.ffn_gate_exps.weight", gate, experts);
+  layer.up_exps = AsTensor("blk.0.ffn_up_exps.weight", up, experts);
+  layer.down_exps = AsTensor("blk.0.ffn_down_exps.weight", down, experts);
+  model.layers.push_back(layer);
+  const HipProjections proj(model);
+
+  for (const int expert : {0, 5, 7}) {
+    for (const int tokens : {1, 4}) {
+      const auto e = static_cast<std::size_t>(expert);
+      const auto x = RandomActivations(static_cast<std::size_t>(tokens) * hidden, rng);
+      const auto want = Expected({&gate, &up}, {e * ffn, e * ffn}, {ffn, ffn}, x, tokens);
+      std::vector<float> got(want.size());
+      proj.ApplyExpert(Stage::kExpertIn, 0, expert, x.data(), tokens, got.data());
+      double err = RelL2(got, want);
+      Report("kExpertIn expert " + std::to_string(expert) + " tokens=" + std::to_string(tokens),
+             err <= kTolerance, err);
+      const auto a = RandomActivations(static_cast<std::size_t>(tokens) * ffn, rng);
+      const auto want_down = Expected({&down}, {e * hidden}, {hidden}, a, tokens);
+      std::vector<float> got_down(want_down.size());
+      proj.ApplyExpert(Stage::kExpertDown, 0, expert, a.data(), tokens, got_down.data());
+      err = RelL2(got_down, want_down);
+      Report("kExpertDown expert " + std::to_string(expert) + " tokens=" + std::to_string(tokens),
+             err <= kTolerance, err);
+    }
+  }
+
+  // Route + the routed FFN against the checker's Reference::Ffn restatement.
+  const int tokens = 6;
+  const auto logits = RandomActivations(static_cast<std::size_t>(tokens) * experts, rng);
+  const auto x = RandomActivations(static_cast<std::size_t>(tokens) * hidden, rng, 0.05f);
+  std::vector<int> chosen(tokens * top), want_chosen(tokens * top);
+  std::vector<float> weights(tokens * top), want_weights(tokens * top);
+  std::vector<float> y(tokens * hidden), want_y(tokens * hidden);
+  proj.Route(logits.data(), tokens, top, chosen.data(), weights.data());
+  gufo_oracle_moe_ffn(gate.bytes.data(), gate.type, up.bytes.data(), up.type, down.bytes.data(),
+                      down.type, experts, static_cast<int>(hidden), static_cast<int>(ffn),
+                      logits.data(), x.data(), tokens, top, want_chosen.data(),
+                      want_weights.data(), want_y.data(), 1, 4);
+  Report("Route indices identical", chosen == want_chosen);
+  Report("Route weights", RelL2(weights, want_weights) <= 1e-6, RelL2(weights, want_weights));
+  proj.RoutedFfn(0, x.data(), tokens, chosen.data(), weights.data(), top, y.data());
+  Report("RoutedFfn", RelL2(y, want_y) <= kTolerance, RelL2(y, want_y));
+
+  std::vector<float> scratch(4096);
+  Report("expert out of range throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.ApplyExpert(Stage::kExpertIn, 0, experts, x.data(), 1, scratch.data());
+         }));
+  Report("ApplyExpert with a dense stage throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.ApplyExpert(Stage::kFfnIn, 0, 0, x.data(), 1, scratch.data());
+         }));
+  ModelTensors bad = model;
+  bad.layers[0].down_exps.shape = {ffn, hidden, 4};
+  Report("expert tensor with the wrong expert count throws std::runtime_error",
+         Throws<std::runtime_error>([&] { HipProjections p(bad); }));
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  if (argc > 1 && std::string(argv[1]) == "--no-device") return RunNoDevice();
+  std::mt19937 rng(20261105);
+  try {
+    RunDense(rng);
+    RunMoe(rng);
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "FAIL: unexpected exception: %s\n", e.what());
+    return 1;
+  }
+  if (g_failures != 0) {
+    std::fprintf(stderr, "FAIL: %d cases\n", g_failures);
+    return 1;
+  }
+  std::puts("PASS");
+  return 0;
+}
