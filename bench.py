@@ -26,6 +26,12 @@ import __graft_entry__ as entry
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0  # dense fp16 / bf16
+# HBM bytes one lm_head launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (`bench.py --counters`), each scaled by what the same counter reads for the 256 MiB
+# read / write probe: 255,457,451 fetched + 613,936 written, 1.0008 x the algorithmic
+# 255,868,416.  Counters cannot be read from inside this process; re-measure with the
+# two commands in profiles/kquant_gemv_decode_set_hbm_traffic.md after a kernel change.
+LM_HEAD_TRAFFIC_BYTES = 256071387
 
 
 def parse_args():
@@ -39,7 +45,30 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--details", action="store_true",
                     help="also time every stage and the other configurations (stderr)")
+    ap.add_argument("--counters", action="store_true",
+                    help="for a `rocprofv3 --pmc` run: a few plain launches of every decode "
+                         "stage plus the read and write probes (known byte counts that "
+                         "calibrate the memory counters), no timing")
     return ap.parse_args()
+
+
+def run_counters(capi, cfg, decode):
+    """Plain (unrecorded) launches, so that a counter run attributes every dispatch."""
+    window = 256 << 20
+    buf = capi.DeviceBuffer(window)
+    sink = capi.DeviceBuffer(64)
+    for _ in range(3):
+        capi.write_probe_dev(buf, window)
+    for _ in range(3):
+        capi.read_probe_dev(buf, window, sink)
+    capi.synchronize()
+    for stage in cfg.CONFIG2_STAGES:
+        for i in range(6):
+            decode.stage(stage, i)
+    capi.synchronize()
+    print(json.dumps({"counters_run": {"probe_bytes": window,
+                                       "launches_per_stage": 6,
+                                       "stages": list(cfg.CONFIG2_STAGES)}}))
 
 
 def log(*args):
@@ -306,6 +335,10 @@ def main():
     log(f"weights resident: {args.layer_copies} layer copies, {args.lm_head_copies} "
         f"lm_head copies ({time.perf_counter() - t0:.1f} s)")
 
+    if args.counters:
+        run_counters(capi, cfg, decode)
+        return
+
     set_bytes = cfg.config2_bytes()
     n_graphs = max(args.layer_copies, args.lm_head_copies)
     n_graphs = args.layer_copies * args.lm_head_copies // np.gcd(args.layer_copies,
@@ -359,7 +392,7 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "us_per_launch": round(ms_head * 1e3, 3),
             "bytes_per_launch": head_bytes,
-            "traffic": None,
+            "traffic": LM_HEAD_TRAFFIC_BYTES,
         },
     }
 

@@ -104,6 +104,7 @@ SIGNATURES = {
     "gufo_hip_timer_begin": (C.c_int, []),
     "gufo_hip_timer_end": (C.c_int, [C.POINTER(C.c_float)]),
     "gufo_hip_read_probe_dev": (C.c_int, [_P, _SZ, _P]),
+    "gufo_hip_write_probe_dev": (C.c_int, [_P, _SZ]),
 }
 
 _lib = None
@@ -382,6 +383,12 @@ def read_probe_dev_at(src: DeviceBuffer, offset: int, nbytes: int, sink: DeviceB
         raise ValueError("probe window outside the buffer")
     _check(load_library().gufo_hip_read_probe_dev(C.c_void_p(src.ptr + offset), nbytes,
                                                   C.c_void_p(sink.ptr)))
+
+
+def write_probe_dev(dst: DeviceBuffer, nbytes: int) -> None:
+    if nbytes > dst.nbytes:
+        raise ValueError("probe window outside the buffer")
+    _check(load_library().gufo_hip_write_probe_dev(C.c_void_p(dst.ptr), nbytes))
 
 
 def read_probe_dev(src: DeviceBuffer, nbytes: int, sink: DeviceBuffer) -> None:

@@ -90,7 +90,25 @@ __global__ __launch_bounds__(256) void ReadProbe(const U32x4* __restrict__ src,
   if (acc == 0x9E3779B9u) *sink = acc;
 }
 
+__global__ __launch_bounds__(256) void WriteProbe(U32x4* __restrict__ dst, size_t n_vec) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+  const U32x4 value = {0x3F800000u, 0x3F800000u, 0x3F800000u, 0x3F800000u};
+  for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n_vec; i += stride) {
+    dst[i] = value;
+  }
+}
+
 }  // namespace
+
+hipError_t LaunchWriteProbe(void* dst, size_t bytes, hipStream_t stream) {
+  const size_t n_vec = bytes / 16;
+  if (n_vec == 0) return hipSuccess;
+  size_t blocks = (n_vec + 256 * 4 - 1) / (256 * 4);
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  hipLaunchKernelGGL(WriteProbe, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, stream,
+                     static_cast<U32x4*>(dst), n_vec);
+  return hipGetLastError();
+}
 
 hipError_t LaunchArgmax(const float* v, size_t n, void* scratch, int64_t* out,
                         hipStream_t stream) {

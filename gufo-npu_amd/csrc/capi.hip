@@ -910,4 +910,14 @@ int gufo_hip_read_probe_dev(const void* src_dev, size_t bytes, uint32_t* sink_de
   return GUFO_HIP_OK;
 }
 
+int gufo_hip_write_probe_dev(void* dst_dev, size_t bytes) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (dst_dev == nullptr || !Aligned16(dst_dev)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "write probe: null or unaligned buffer");
+  }
+  GUFO_HIP_TRY(gufo::LaunchWriteProbe(dst_dev, bytes, g_state.stream));
+  return GUFO_HIP_OK;
+}
+
 }  // extern "C"

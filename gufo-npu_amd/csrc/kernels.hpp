@@ -122,4 +122,7 @@ hipError_t LaunchArgmax(const float* v, size_t n, void* scratch, int64_t* out,
 hipError_t LaunchReadProbe(const void* src, size_t bytes, uint32_t* sink,
                            hipStream_t stream);
 
+// Streaming write of `bytes` (multiple of 16) of a constant.
+hipError_t LaunchWriteProbe(void* dst, size_t bytes, hipStream_t stream);
+
 }  // namespace gufo

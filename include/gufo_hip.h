@@ -207,6 +207,11 @@ int gufo_hip_timer_end(float* milliseconds);
  * *sink_dev is written only if a lane's xor of its data equals a magic constant
  * (that keeps the loads alive without timing a store). */
 int gufo_hip_read_probe_dev(const void* src_dev, size_t bytes, uint32_t* sink_dev);
+/* The write-side twin (the reference's bw_memcpy probe, src/npu/device.hpp:58-66):
+ * a plain streaming store of a constant over `bytes` of device memory.  Together
+ * the two probes calibrate the memory-traffic counters of a profiler run: both move
+ * a known number of bytes. */
+int gufo_hip_write_probe_dev(void* dst_dev, size_t bytes);
 
 #ifdef __cplusplus
 }
