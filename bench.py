@@ -304,7 +304,7 @@ def cpu_baseline(cfg, decode, seconds):
     t0 = time.perf_counter()
     one_set()
     probe = time.perf_counter() - t0
-    reps = int(max(3, min(400, seconds / max(probe, 1e-6))))
+    reps = int(max(3, min(5000, seconds / max(probe, 1e-6))))
     t0 = time.perf_counter()
     for _ in range(reps):
         one_set()

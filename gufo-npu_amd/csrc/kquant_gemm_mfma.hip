@@ -3,31 +3,43 @@
 // tokens = m (src/models/qwen35/gguf_projections.cpp:239-286 of the reference), the
 // shape the reference's NPU serves with its prefill GEMM (src/npu/gemm.hpp:99-105).
 //
-// The weights are never dequantized to memory.  What the matrix cores multiply are
-// exact 16-bit operands:
+// The weights are dequantized in the kernel, in registers, to 16-bit operands and
+// never written to memory:
 //
-//   weight[r][k] = d * (sc_j * q) - dmin * m_j        (j = sub-block of k)
+//   weight[r][k] = d * sc_j * q - dmin * m_j          (j = sub-block of k)
 //
-//   * sc_j * q is an integer <= 63 * 15 = 945, exact in fp16 (11-bit significand) -
-//     it would not be in bf16 (8 bits), and rounding the dequantized weight itself to
-//     bf16 costs 1.7e-3 relative L2 on this workload, above the 1e-3 this kernel is
-//     held to.  The bf16 activations convert to fp16 without loss (8-bit significand;
-//     magnitudes below 2^-24 flush, far below anything that matters).
-//   * v_mfma_f32_32x32x16_f16 accumulates sum_k (sc*q) * a over one super-block (16
-//     instructions) in fp32; the block scale d, one value per weight row = per lane
-//     of the accumulator layout, is applied once per super-block with one fma per
-//     accumulator register.
-//   * The minimum term needs sum over each sub-block of a, S[t][j].  A pre-pass
-//     writes the activations as fp16 together with S split in two fp16 halves
-//     (hi + lo, 22 bits), so the term is one more MFMA per super-block: K = 16 =
-//     8 sub-blocks x {hi, lo} against the 6-bit minimums m_j, scaled by dmin.
+//   * 16-bit means fp16, not bf16: rounding the dequantized weight to bf16 (8-bit
+//     significand) costs 1.7e-3 relative L2 on this workload, above the 1e-3 this
+//     kernel is held to; fp16 (11 bits) costs 1.4e-4.  The bf16 activations convert
+//     to fp16 without loss (a pre-pass; magnitudes above 65504 saturate, below 2^-24
+//     flush).
+//   * The 4-bit code becomes the fp16 number 1024 + q by a byte permute
+//     (0x6400 | q), and one fp32 fma with fp16 input and fp16 result
+//     (v_fma_mix) produces the weight with a single rounding:
+//     (1024 + q) * (d sc_j) - (1024 d sc_j + dmin m_j).  d sc_j is exact in fp32
+//     (11 x 6 bits); the offset is rounded to fp32 once per sub-block, 2^-14 of a
+//     quantization step.
+//   * v_mfma_f32_32x32x16_f16 accumulates in fp32 over the whole row.
 //
-// Decomposition: a workgroup of 4 waves computes 128 tokens x 128 weight rows.  The
-// activation tile of one super-block (128 x 272 fp16) is staged in LDS and shared;
-// each wave owns 32 weight rows, reads their packed blocks straight into registers
-// one super-block ahead, converts them to operand fragments on the fly (a byte
-// permute and one packed fp16 fma per two weights) and multiplies them with the four
-// 32-token tiles.
+// Decomposition: a workgroup of 4 waves computes 128 tokens x 128 weight rows, two
+// workgroups to a CU.  The activation tile of half a super-block (128 tokens x 128
+// fp16 = 32 KB) goes from global memory straight into LDS (global_load_lds_dwordx4),
+// double-buffered, one half ahead of the matrix cores; each wave owns 32 weight rows,
+// reads their packed blocks into registers one super-block ahead, builds the operand
+// fragments on the fly and multiplies them with the four 32-token tiles.
+//
+// The matrix instruction does not care which k a lane's 8 values belong to as long as
+// both operands agree, so k is dealt to lanes the way the packed block likes it: of
+// each 64 values (32 bytes of codes: low nibbles one sub-block, high nibbles the
+// next), lane half u owns bytes 16 u .. 16 u + 15 - one 16-byte load - and its four
+// steps take (low, first 8), (low, second 8), (high, first 8), (high, second 8).
+//
+// Workgroups are numbered so that each of the 8 XCDs (which take workgroups
+// round-robin) owns a band of weight-row tiles - its slice of the packed matrix
+// stays in that XCD's L2 - and walks the token tiles in order, so the workgroups
+// running together share activation tiles.
+#include <type_traits>
+
 #include "kernels.hpp"
 #include "kquant_common.hpp"
 
@@ -37,121 +49,178 @@ namespace {
 typedef _Float16 Half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 Half2 __attribute__((ext_vector_type(2)));
 typedef float Float16v __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* LdsPointer;
 
 constexpr int kGemmThreads = 256;
-constexpr int kTileTokens = 128;  // BM
-constexpr int kTileRows = 128;    // BN
-constexpr int kBlockHalfs = 272;  // 256 activations + 8 sub-block sums hi + 8 lo
-constexpr int kLdsPitch = 280;    // halfs per token row in LDS: 560 B, an odd number of
-                                  // 16-byte units, so 8 consecutive rows hit 8 bank groups
+constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kTileTokens = 128;
+constexpr int kTileRows = 32 * kGemmWaves;
+constexpr int kRowBytes = 256;                            // one token's half super-block as fp16
+constexpr int kStageBytes = kTileTokens * kRowBytes;      // 32 KB
+constexpr int kCopiesPerWave = kStageBytes / 1024 / kGemmWaves;  // 1 KB per wave instruction
 constexpr int kQ4Block = 144;
+constexpr int kXcds = 8;
 
-// ---- pre-pass: bf16 activations -> fp16 + sub-block sums ------------------------
-// out[t][b][0..255] = a[t][256 b + i] as fp16, out[t][b][256 + j] = hi(S_j),
-// out[t][b][264 + j] = lo(S_j), S_j = sum of the 32 activations of sub-block j (fp32).
-// One wave per (token, super-block); lane l converts values 4l..4l+3.
-__global__ __launch_bounds__(256) void PrepareActivations(const uint16_t* __restrict__ a,
-                                                          uint32_t tokens, uint32_t nb,
-                                                          _Float16* __restrict__ out) {
-  const uint32_t item = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (item >= tokens * nb) return;
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t t = item / nb;
-  const uint32_t b = item - t * nb;
-  const U32x2 raw =
-      *reinterpret_cast<const U32x2*>(a + (static_cast<size_t>(t) * nb + b) * 256 + 4 * lane);
-  float v[4];
-  v[0] = __uint_as_float(raw.x << 16);
-  v[1] = __uint_as_float(raw.x & 0xFFFF0000u);
-  v[2] = __uint_as_float(raw.y << 16);
-  v[3] = __uint_as_float(raw.y & 0xFFFF0000u);
-  _Float16* dst = out + (static_cast<size_t>(t) * nb + b) * kBlockHalfs;
-  Half2 h01 = {static_cast<_Float16>(v[0]), static_cast<_Float16>(v[1])};
-  Half2 h23 = {static_cast<_Float16>(v[2]), static_cast<_Float16>(v[3])};
-  U32x2 packed = {__builtin_bit_cast(uint32_t, h01), __builtin_bit_cast(uint32_t, h23)};
-  *reinterpret_cast<U32x2*>(dst + 4 * lane) = packed;
-  // Sub-block j = lanes 8j..8j+7: sum in a fixed order.
-  float s = (v[0] + v[1]) + (v[2] + v[3]);
-  s += __shfl_xor(s, 1, 64);
-  s += __shfl_xor(s, 2, 64);
-  s += __shfl_xor(s, 4, 64);
-  if ((lane & 7) == 0) {
-    const _Float16 hi = static_cast<_Float16>(s);
-    const _Float16 lo = static_cast<_Float16>(s - static_cast<float>(hi));
-    dst[256 + (lane >> 3)] = hi;
-    dst[264 + (lane >> 3)] = lo;
+// ---- pre-pass: bf16 activations -> fp16, same [token][k] layout -------------------
+__global__ __launch_bounds__(256) void PrepareActivations(const U32x4* __restrict__ a,
+                                                          size_t octets,
+                                                          U32x4* __restrict__ out) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= octets) return;
+  const U32x4 raw = a[i];
+  const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t packed[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    float lo = __uint_as_float(in[p] << 16);
+    float hi = __uint_as_float(in[p] & 0xFFFF0000u);
+    lo = __builtin_fminf(__builtin_fmaxf(lo, -65504.0f), 65504.0f);
+    hi = __builtin_fminf(__builtin_fmaxf(hi, -65504.0f), 65504.0f);
+    const Half2 h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    packed[p] = __builtin_bit_cast(uint32_t, h);
   }
+  out[i] = U32x4{packed[0], packed[1], packed[2], packed[3]};
 }
 
 // ---- the product ------------------------------------------------------------------
 
-// One weight row's packed super-block as this lane reads it.  Lane (n, u) = (lane%32,
-// lane/32) owns, of each MFMA step s (16 k-values), the 8 values k = 16 s + 8 u .. +8
-// of row n: sub-block s/2, bytes 32 (s/4) + 16 (s%2) + 8 u .. +8 of qs, low nibbles
-// for even s/2 and high nibbles for odd.  Over a block that is 8 pieces of 8 bytes.
+// Where the 16-byte piece p (0..15) of token row t sits inside the row's 256 bytes of
+// LDS: slot p ^ Swizzle(t).  Rows are one bank sweep apart, so the slot alone decides
+// the banks; a wave reads piece (c | 2 u) of rows n = 0..31, and the xor makes the 16
+// slots of rows n..n+15 (either u) and of rows n..n+7 (both u) all different.
+__device__ __forceinline__ uint32_t Swizzle(uint32_t t) {
+  return (t & 1u) | (((t >> 1) & 3u) << 2) | (((t >> 3) & 1u) << 1);
+}
+
+// One weight row's packed super-block as this lane reads it: lane (n, u) = (lane % 32,
+// lane / 32) takes bytes 16 u .. 16 u + 15 of each 32 bytes of codes of row n.
 struct PackedRow {
   U32x4 header;     // d, dmin, 12 scale bytes
-  U32x2 piece[8];   // piece[2 p + h] = qs[32 p + 16 h + 8 u .. +8)
+  U32x4 codes[4];   // codes[p] = qs[32 p + 16 u .. +16)
 
   __device__ __forceinline__ void Load(const uint8_t* blk, uint32_t u) {
     header = Load16(blk);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      piece[i] = *reinterpret_cast<const U32x2*>(blk + 16 + 32 * (i >> 1) + 16 * (i & 1) + 8 * u);
-    }
-  }
-  __device__ __forceinline__ void Clear() {
-    header = U32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) piece[i] = U32x2{0, 0};
+    for (int p = 0; p < 4; ++p) codes[p] = Load16(blk + 16 + 32 * p + 16 * u);
   }
 };
 
-// Two 4-bit codes (bytes b0, b1 of `nibbles`, each 0..15) times the integer scale, as
-// two exact fp16: (1024 + q) * sc - 1024 * sc with 0x6400 | q = 1024 + q.
-__device__ __forceinline__ uint32_t ScaledPair(uint32_t nibbles, uint32_t selector,
-                                               Half2 scale, Half2 offset) {
+// Two 4-bit codes (bytes of `nibbles` picked by `selector`, each 0..15) dequantized to
+// two fp16: the permute builds 0x6400 | q = 1024 + q, the fma runs in fp32.
+__device__ __forceinline__ uint32_t DequantPair(uint32_t nibbles, uint32_t selector, float scale,
+                                                float offset) {
   const uint32_t biased = __builtin_amdgcn_perm(0x64646464u, nibbles, selector);
   const Half2 h = __builtin_bit_cast(Half2, biased);
-  const Half2 r = __builtin_elementwise_fma(h, scale, offset);
+  Half2 r;
+  r[0] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>(h[0]), scale, offset));
+  r[1] = static_cast<_Float16>(__builtin_fmaf(static_cast<float>(h[1]), scale, offset));
   return __builtin_bit_cast(uint32_t, r);
 }
 
-// The B operand of step s: 8 values (sc_j * q) as fp16 for this lane.
+// Step s = 4 p + 2 high + half of a super-block: this lane's 8 dequantized values,
+// k = 64 p + 32 high + 16 u + 8 half .. +8 of sub-block 2 p + high.
 __device__ __forceinline__ Half8 WeightFragment(const PackedRow& row, int s,
-                                                const uint32_t (&sc)[8]) {
-  const int j = s >> 1;                       // sub-block
-  const U32x2 bytes = row.piece[2 * (s >> 2) + (s & 1)];
+                                                const float (&scale)[8],
+                                                const float (&offset)[8]) {
+  const int p = s >> 2;
+  const int j = s >> 1;
+  const uint32_t b0 = (s & 1) ? row.codes[p].z : row.codes[p].x;
+  const uint32_t b1 = (s & 1) ? row.codes[p].w : row.codes[p].y;
   const uint32_t shift = (j & 1) ? 4 : 0;
-  const uint32_t n0 = (bytes.x >> shift) & 0x0F0F0F0Fu;
-  const uint32_t n1 = (bytes.y >> shift) & 0x0F0F0F0Fu;
-  const _Float16 scale = static_cast<_Float16>(static_cast<float>(sc[j]));
-  const Half2 scale2 = {scale, scale};
-  const _Float16 off = static_cast<_Float16>(-1024.0f * static_cast<float>(sc[j]));
-  const Half2 off2 = {off, off};
+  const uint32_t n0 = (b0 >> shift) & 0x0F0F0F0Fu;
+  const uint32_t n1 = (b1 >> shift) & 0x0F0F0F0Fu;
   // perm selectors: result bytes [3..0] = [0x64, q_hi, 0x64, q_lo]; source 1 (nibbles)
   // holds bytes 0-3, source 0 (the constant) bytes 4-7.
   U32x4 out;
-  out.x = ScaledPair(n0, 0x04010400u, scale2, off2);  // codes 0, 1
-  out.y = ScaledPair(n0, 0x04030402u, scale2, off2);  // codes 2, 3
-  out.z = ScaledPair(n1, 0x04010400u, scale2, off2);  // codes 4, 5
-  out.w = ScaledPair(n1, 0x04030402u, scale2, off2);  // codes 6, 7
+  out.x = DequantPair(n0, 0x04010400u, scale[j], offset[j]);  // codes 0, 1
+  out.y = DequantPair(n0, 0x04030402u, scale[j], offset[j]);  // codes 2, 3
+  out.z = DequantPair(n1, 0x04010400u, scale[j], offset[j]);  // codes 4, 5
+  out.w = DequantPair(n1, 0x04030402u, scale[j], offset[j]);  // codes 6, 7
   return __builtin_bit_cast(Half8, out);
 }
 
-__global__ __launch_bounds__(kGemmThreads) void KquantGemmKernel(
-    const uint8_t* __restrict__ w, uint32_t rows, uint32_t nb,
-    const _Float16* __restrict__ a16, uint32_t tokens, float* __restrict__ c) {
-  extern __shared__ __align__(16) _Float16 tile[];  // kTileTokens x kLdsPitch
+// The 16-byte piece of a token's half super-block that step s (0..7 within the half)
+// reads for lane half u = 0; lane half 1 reads the piece 2 further.
+__device__ __forceinline__ constexpr uint32_t StepPiece(int s) {
+  return 8u * ((s >> 2) & 1) + 4u * ((s >> 1) & 1) + (s & 1);
+}
+
+struct GemmShape {
+  uint32_t rows;
+  uint32_t nb;           // super-blocks per row
+  uint32_t tokens;
+  uint32_t row_tiles;
+  uint32_t token_tiles;
+  uint32_t band;         // weight-row tiles per band
+  uint32_t per_xcd;      // workgroups each XCD takes
+  uint32_t total;        // bands * token_tiles * band
+};
+
+// Waits until at most `pending` of this wave's vector-memory operations are
+// outstanding (they retire in order).
+template <int kPending>
+__device__ __forceinline__ void WaitVectorMemory() {
+  if constexpr (kPending == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    static_assert(kPending == 5, "one packed row is 5 loads");
+    asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  }
+}
+
+// The workgroup barrier alone.  __syncthreads() adds a release fence that drains every
+// vector-memory operation of the wave, the weight prefetch included; here the waits
+// that matter are explicit: each wave waits for its own copies into LDS before the
+// barrier, and has consumed its LDS reads of the other stage by then.
+__device__ __forceinline__ void TileBarrier() {
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// Two workgroups share a CU (2 x 64 KB of LDS, 2 waves per SIMD).
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
+                 float* __restrict__ c, GemmShape shape) {
+  extern __shared__ __align__(1024) uint8_t stages[];  // 2 x kStageBytes
+  // Workgroup -> tile.  XCD x takes positions [x per_xcd, (x+1) per_xcd) of the order
+  // (band, token tile, row tile within the band).
+  const uint32_t position = (blockIdx.x % kXcds) * shape.per_xcd + blockIdx.x / kXcds;
+  if (position >= shape.total) return;
+  const uint32_t within = position % shape.band;
+  const uint32_t token_tile = (position / shape.band) % shape.token_tiles;
+  const uint32_t row_tile = position / (shape.band * shape.token_tiles) * shape.band + within;
+  if (row_tile >= shape.row_tiles) return;
+
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63;
   const uint32_t wave = tid >> 6;
   const uint32_t n = lane & 31;
   const uint32_t u = lane >> 5;
-  const uint32_t token0 = blockIdx.y * kTileTokens;
-  const uint32_t row = blockIdx.x * kTileRows + wave * 32 + n;
-  const bool row_valid = row < rows;
-  const uint8_t* row_ptr = w + static_cast<size_t>(row_valid ? row : 0) * nb * kQ4Block;
+  const uint32_t nb = shape.nb;
+  const uint32_t token0 = token_tile * kTileTokens;
+  const uint32_t row = row_tile * kTileRows + wave * 32 + n;
+  const bool row_valid = row < shape.rows;
+  const uint8_t* row_ptr = w + static_cast<size_t>(row_valid ? row : shape.rows - 1) * nb * kQ4Block;
+
+  // Copies global -> LDS.  Wave instruction i of this wave fills the 1 KB holding token
+  // rows 4 c .. 4 c + 3 (c = wave * kCopiesPerWave + i); lane l supplies LDS slot l % 16
+  // of row 4 c + l / 16, that is piece slot ^ Swizzle(row) of the token's half block.
+  // Rows past the last token repeat it; their products are not stored.
+  uint32_t copy_piece[kCopiesPerWave];  // in 16-byte pieces from a16, half block 0
+#pragma unroll
+  for (int i = 0; i < kCopiesPerWave; ++i) {
+    const uint32_t t = 4 * (wave * kCopiesPerWave + i) + (lane >> 4);
+    const uint32_t token = min(token0 + t, shape.tokens - 1);
+    copy_piece[i] = token * (nb * 32) + ((lane & 15u) ^ Swizzle(t & 15u));
+  }
+  auto copy_stage = [&](uint32_t half_block, uint32_t stage) {
+#pragma unroll
+    for (int i = 0; i < kCopiesPerWave; ++i) {
+      const uint8_t* src = a16 + (static_cast<size_t>(copy_piece[i]) + half_block * 16) * 16;
+      uint8_t* dst = stages + stage * kStageBytes + (wave * kCopiesPerWave + i) * 1024;
+      __builtin_amdgcn_global_load_lds(src, (LdsPointer)dst, 16, 0, 0);
+    }
+  };
 
   Float16v acc[4];
 #pragma unroll
@@ -160,75 +229,97 @@ __global__ __launch_bounds__(kGemmThreads) void KquantGemmKernel(
     for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
   }
 
+  copy_stage(0, 0);
   PackedRow next;
-  if (row_valid) {
-    next.Load(row_ptr, u);
-  } else {
-    next.Clear();
-  }
+  next.Load(row_ptr, u);
 
-  for (uint32_t b = 0; b < nb; ++b) {
-    const PackedRow cur = next;
-    if (b + 1 < nb && row_valid) next.Load(row_ptr + static_cast<size_t>(b + 1) * kQ4Block, u);
+  // This lane's activation fragment of step s, token tile m: piece StepPiece(s) | 2 u of
+  // row 32 m + n, at slot StepPiece(s) ^ flip.
+  const uint32_t flip = Swizzle(n & 15u) ^ (u << 1);
+  const uint32_t read_base = n * kRowBytes;
 
-    // Stage the activation tile of this super-block: 128 rows of 272 halfs = 34 pieces
-    // of 16 bytes per row.
-    __syncthreads();
-    for (uint32_t i = tid; i < kTileTokens * 34; i += kGemmThreads) {
-      const uint32_t t = i / 34;
-      const uint32_t piece = i - t * 34;
-      U32x4 v = {0, 0, 0, 0};
-      if (token0 + t < tokens) {
-        v = *reinterpret_cast<const U32x4*>(
-            a16 + (static_cast<size_t>(token0 + t) * nb + b) * kBlockHalfs + piece * 8);
-      }
-      *reinterpret_cast<U32x4*>(tile + t * kLdsPitch + piece * 8) = v;
-    }
-    __syncthreads();
+  PackedRow cur;
+  float scale[8];
+  float offset[8];
 
-    const float d = HalfBitsToFloat(cur.header.x & 0xFFFFu);
-    const float dmin = HalfBitsToFloat(cur.header.x >> 16);
-    uint32_t sc[8];
-    uint32_t mn[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      ScaleMinK4(cur.header.y, cur.header.z, cur.header.w, j, &sc[j], &mn[j]);
-    }
-
-    Float16v part[4];
+  // One half super-block: 8 steps on `stage`, both operands one step ahead of the
+  // matrix cores - while step s multiplies, the activation fragments of step s + 1 are
+  // on their way from LDS and its weight fragment is being dequantized.
+  auto multiply_half = [&](uint32_t stage, auto half_tag) {
+    constexpr int kHalf = decltype(half_tag)::value;
+    const uint8_t* tile = stages + stage * kStageBytes + read_base;
+    Half8 af[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) part[m][i] = 0.0f;
+      af[m] = *reinterpret_cast<const Half8*>(tile + ((StepPiece(0) ^ flip) << 4) +
+                                              m * 32 * kRowBytes);
     }
+    Half8 bf = WeightFragment(cur, 8 * kHalf, scale, offset);
 #pragma unroll
-    for (int s = 0; s < 16; ++s) {
-      const Half8 bf = WeightFragment(cur, s, sc);
+    for (int s = 0; s < 8; ++s) {
+      Half8 af_next[4];
+      Half8 bf_next;
+      if (s + 1 < 8) {
+        const uint8_t* at = tile + ((StepPiece(s + 1) ^ flip) << 4);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          af_next[m] = *reinterpret_cast<const Half8*>(at + m * 32 * kRowBytes);
+        }
+      }
+      // Nothing moves across: the reads of step s + 1 are issued before step s multiplies.
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < 8) bf_next = WeightFragment(cur, 8 * kHalf + s + 1, scale, offset);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        const Half8 af = *reinterpret_cast<const Half8*>(tile + (m * 32 + n) * kLdsPitch +
-                                                         16 * s + 8 * u);
-        part[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, part[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[m], bf, acc[m], 0, 0, 0);
+      }
+      // Within the step: each matrix instruction followed by a quarter of the next
+      // weight fragment's dequantization.
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < 8) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) af[m] = af_next[m];
+        bf = bf_next;
       }
     }
-    // The minimum term: k = 8 u + j pairs m_j with hi(S_j) (u = 0) or lo(S_j) (u = 1).
-    Half8 mins;
+  };
+
+  for (uint32_t b = 0; b < nb; ++b) {
+    const bool more = b + 1 < nb;
+    // First half.  Everything in flight (stage 0's copies, this block's weights) has
+    // landed, for every wave, and every wave is done reading stage 1.
+    WaitVectorMemory<0>();
+    TileBarrier();
+    cur = next;
+    copy_stage(2 * b + 1, 1);
+    __builtin_amdgcn_sched_barrier(0);  // the wait below counts on this issue order
+    if (more) next.Load(row_ptr + static_cast<size_t>(b + 1) * kQ4Block, u);
+    const float d = HalfBitsToFloat(cur.header.x & 0xFFFFu);
+    const float dmin = HalfBitsToFloat(cur.header.x >> 16);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) mins[j] = static_cast<_Float16>(static_cast<float>(mn[j]));
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const Half8 sums = *reinterpret_cast<const Half8*>(tile + (m * 32 + n) * kLdsPitch + 256 +
-                                                         8 * u);
-      Float16v zero;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
-      const Float16v min_part = __builtin_amdgcn_mfma_f32_32x32x16_f16(sums, mins, zero, 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        acc[m][i] = __builtin_fmaf(d, part[m][i], acc[m][i]);
-        acc[m][i] = __builtin_fmaf(-dmin, min_part[i], acc[m][i]);
-      }
+    for (int j = 0; j < 8; ++j) {
+      uint32_t sc, mn;
+      ScaleMinK4(cur.header.y, cur.header.z, cur.header.w, j, &sc, &mn);
+      scale[j] = d * static_cast<float>(sc);
+      offset[j] = __builtin_fmaf(-dmin, static_cast<float>(mn), -1024.0f * scale[j]);
     }
+    multiply_half(0, std::integral_constant<int, 0>{});
+
+    // Second half.  Stage 1's copies were issued before the next block's weights, which
+    // may stay in flight.
+    if (more) {
+      WaitVectorMemory<5>();
+    } else {
+      WaitVectorMemory<0>();
+    }
+    TileBarrier();
+    if (more) copy_stage(2 * b + 2, 0);
+    multiply_half(1, std::integral_constant<int, 1>{});
   }
 
   // Accumulator register i of tile m holds token 8 (i/4) + 4 u + i%4 and weight row n.
@@ -238,7 +329,7 @@ __global__ __launch_bounds__(kGemmThreads) void KquantGemmKernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const uint32_t t = token0 + m * 32 + 8 * (i >> 2) + 4 * u + (i & 3);
-        if (t < tokens) c[static_cast<size_t>(t) * rows + row] = acc[m][i];
+        if (t < shape.tokens) c[static_cast<size_t>(t) * shape.rows + row] = acc[m][i];
       }
     }
   }
@@ -247,35 +338,37 @@ __global__ __launch_bounds__(kGemmThreads) void KquantGemmKernel(
 }  // namespace
 
 size_t GemmWorkspaceBytes(size_t tokens, uint32_t blocks_per_row) {
-  return tokens * blocks_per_row * kBlockHalfs * sizeof(_Float16);
+  return tokens * blocks_per_row * 256 * sizeof(_Float16);
 }
 
 hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
                          const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
                          hipStream_t stream) {
   if (rows == 0 || tokens == 0) return hipSuccess;
-  if (blocks_per_row == 0 || tokens > 0x7FFFFFFFull / blocks_per_row) {
+  // Activation pieces are addressed with 32 bits.
+  if (blocks_per_row == 0 || tokens > 0x7FFFFFFFull / (32ull * blocks_per_row)) {
     return hipErrorInvalidValue;
   }
-  _Float16* a16 = static_cast<_Float16*>(workspace);
-  const uint32_t items = static_cast<uint32_t>(tokens) * blocks_per_row;
-  hipLaunchKernelGGL(PrepareActivations, dim3((items + 3) / 4), dim3(256), 0, stream, a_bf16,
-                     static_cast<uint32_t>(tokens), blocks_per_row, a16);
+  const size_t octets = tokens * blocks_per_row * 32;
+  hipLaunchKernelGGL(PrepareActivations, dim3(static_cast<uint32_t>((octets + 255) / 256)),
+                     dim3(256), 0, stream, reinterpret_cast<const U32x4*>(a_bf16), octets,
+                     static_cast<U32x4*>(workspace));
   hipError_t status = hipGetLastError();
   if (status != hipSuccess) return status;
-  const size_t lds_bytes = static_cast<size_t>(kTileTokens) * kLdsPitch * sizeof(_Float16);
-  static bool allowed = false;
-  if (!allowed) {
-    status = hipFuncSetAttribute(reinterpret_cast<const void*>(KquantGemmKernel),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 static_cast<int>(lds_bytes));
-    if (status != hipSuccess) return status;
-    allowed = true;
-  }
-  const dim3 grid((rows + kTileRows - 1) / kTileRows,
-                  static_cast<uint32_t>((tokens + kTileTokens - 1) / kTileTokens));
-  hipLaunchKernelGGL(KquantGemmKernel, grid, dim3(kGemmThreads), lds_bytes, stream, w, rows,
-                     blocks_per_row, a16, static_cast<uint32_t>(tokens), c);
+
+  constexpr size_t lds_bytes = 2 * kStageBytes;
+  GemmShape shape;
+  shape.rows = rows;
+  shape.nb = blocks_per_row;
+  shape.tokens = static_cast<uint32_t>(tokens);
+  shape.row_tiles = (rows + kTileRows - 1) / kTileRows;
+  shape.token_tiles = static_cast<uint32_t>((tokens + kTileTokens - 1) / kTileTokens);
+  shape.band = (shape.row_tiles + kXcds - 1) / kXcds;
+  const uint32_t bands = (shape.row_tiles + shape.band - 1) / shape.band;
+  shape.total = bands * shape.token_tiles * shape.band;
+  shape.per_xcd = (shape.total + kXcds - 1) / kXcds;
+  hipLaunchKernelGGL(KquantGemmKernel, dim3(shape.per_xcd * kXcds), dim3(kGemmThreads), lds_bytes,
+                     stream, w, static_cast<const uint8_t*>(workspace), c, shape);
   return hipGetLastError();
 }
 

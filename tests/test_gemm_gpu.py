@@ -2,7 +2,8 @@
 with the CPU checker and the golden reference slice, through the C-ABI.
 
 Bar: rel-L2 <= 1e-3 against dequantize + double sum over the same bf16 activation
-values (the bar stated for this kernel); in practice the kernel is ~1e-6."""
+values (the bar stated for this kernel).  The kernel rounds each dequantized weight to
+fp16 once (relative 2^-12 at most) and accumulates in fp32, which lands near 1.5e-4."""
 import numpy as np
 import pytest
 
@@ -12,6 +13,7 @@ from gufo_npu_amd import synth
 
 pytestmark = pytest.mark.gpu
 TOLERANCE = 1e-3
+VS_GEMV = 5e-4     # the GEMV kernels are ~1e-7 from the truth, so this bounds the GEMM alone
 
 
 def say(*args):
@@ -38,12 +40,14 @@ def test_gemm_parity_small_and_ragged(hip, oracle, tokens, rows, cols):
     # every row of C is the matrix-vector product of that token
     for t in sorted({0, tokens // 2, tokens - 1}):
         single = hip.gemv([hip.whole(m)], a[t:t + 1], 1)
-        assert oracle.rel_l2(got[t], single[0]) <= 1e-4
+        assert oracle.rel_l2(got[t], single[0]) <= VS_GEMV
     m.destroy()
 
 
 def test_gemm_unit_activations_return_the_weights(hip, oracle):
-    # a = unit vectors (exact in bf16): C[t] is column t of the dequantized matrix.
+    # a = unit vectors (exact in bf16): C[t] is column t of the dequantized matrix, each
+    # weight rounded to fp16 once: off by at most half an fp16 ulp, 2^-11 relative (the
+    # weights here are far above the fp16 subnormal range, where the bound is absolute).
     say("gemm identity")
     rows, cols = 64, 512
     w = synth.kquant_matrix(synth.Q4_K, rows, cols, 99)
@@ -51,7 +55,12 @@ def test_gemm_unit_activations_return_the_weights(hip, oracle):
     bits = synth.bf16_round(np.eye(cols, dtype=np.float32))
     got = hip.gemm_q4k_bf16(m, bits)
     want = np.stack([oracle.dequantize(synth.Q4_K, w[r], cols) for r in range(rows)], axis=1)
-    assert oracle.rel_l2(got, want) <= 1e-6
+    assert got.shape == want.shape
+    # plus the offset 1024 d sc + dmin m rounded to fp32: below 1e-4 of the row's largest
+    slack = 1e-4 * np.abs(want).max(axis=0, keepdims=True)
+    bound = np.maximum(np.abs(want) * 2.0 ** -11, 2.0 ** -25) + slack
+    assert bool(np.all(np.abs(got.astype(np.float64) - want) <= bound))
+    assert oracle.rel_l2(got, want) <= 3e-4
     m.destroy()
 
 
@@ -81,6 +90,6 @@ def test_config5_prefill_projection(hip, oracle):
                          threads=8)
     assert oracle.rel_l2(got[pick], want) <= TOLERANCE
     single = hip.gemv([hip.whole(m)], a[pick], len(pick))
-    assert oracle.rel_l2(got[pick], single) <= 1e-4
+    assert oracle.rel_l2(got[pick], single) <= VS_GEMV
     say("config 5 rel-L2 vs double", oracle.rel_l2(got[pick], want))
     m.destroy()
