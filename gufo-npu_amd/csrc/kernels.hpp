@@ -30,6 +30,7 @@ constexpr size_t kGemvMaxLdsBytes = 160 * 1024;
 
 // The compute-unit count of the device, which sizes the persistent launches.
 void SetGemvComputeUnits(int compute_units);
+int DeviceComputeUnits();
 
 // Token columns one launch can carry for rows of blocks_per_row super-blocks: the
 // quantized activation rows of all columns must fit in LDS together (at most

@@ -853,6 +853,8 @@ void SetGemvComputeUnits(int compute_units) {
   if (compute_units > 0) g_compute_units = compute_units;
 }
 
+int DeviceComputeUnits() { return g_compute_units; }
+
 int GemvMaxTokens(int type, uint32_t blocks_per_row) {
   const size_t per_token = LdsBytes(type, blocks_per_row, 1);
   if (per_token == 0) return 0;
