@@ -296,7 +296,9 @@ int RouteDevLocked(const float* logits, int tokens, int experts, int k, int* ids
   return GUFO_HIP_OK;
 }
 
-int GroupDevLocked(const int* ids, int tokens, int k, int experts,
+// segments_only: the caller reads the segment list, pair_valid and the header, not the
+// per-expert counts, offsets and pair order.
+int GroupDevLocked(const int* ids, int tokens, int k, int experts, bool segments_only,
                    MoeTablePointers* tables) {
   if (tokens < 0 || k <= 0 || experts <= 0) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "group: tokens %d, k %d, experts %d",
@@ -309,9 +311,14 @@ int GroupDevLocked(const int* ids, int tokens, int k, int experts,
                 gufo::kMaxGroupPairs, gufo::kMaxGroupExperts);
   }
   GUFO_TRY(ReserveMoeTables(static_cast<int>(n_pairs > 0 ? n_pairs : 1), experts, tables));
-  GUFO_HIP_TRY(gufo::LaunchMoeGroup(ids, static_cast<int>(n_pairs), experts,
-                                    tokens < kMaxGemvTokens ? (tokens > 0 ? tokens : 1)
-                                                            : kMaxGemvTokens,
+  const int capacity = tokens < kMaxGemvTokens ? (tokens > 0 ? tokens : 1) : kMaxGemvTokens;
+  if (segments_only && n_pairs <= gufo::kMaxSmallGroupPairs) {
+    GUFO_HIP_TRY(gufo::LaunchMoeGroupSmall(ids, static_cast<int>(n_pairs), experts, capacity,
+                                           tables->valid, tables->segments, tables->header,
+                                           g_state.stream));
+    return GUFO_HIP_OK;
+  }
+  GUFO_HIP_TRY(gufo::LaunchMoeGroup(ids, static_cast<int>(n_pairs), experts, capacity,
                                     tables->counts, tables->offsets, tables->pairs,
                                     tables->valid, tables->segments, tables->header,
                                     g_state.stream));
@@ -345,7 +352,7 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   }
   if (!Aligned16(x)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
   MoeTablePointers tables;
-  GUFO_TRY(GroupDevLocked(ids, tokens, k, experts, &tables));
+  GUFO_TRY(GroupDevLocked(ids, tokens, k, experts, true, &tables));
   const size_t n_pairs = static_cast<size_t>(tokens) * k;
   GUFO_TRY(Reserve(&g_state.moe_gate_up, n_pairs * 2 * ffn * sizeof(float)));
   GUFO_TRY(Reserve(&g_state.moe_out, n_pairs * hidden * sizeof(float)));
@@ -720,7 +727,7 @@ int gufo_hip_moe_group(const int* ids_host, int tokens, int k, int experts,
   GUFO_TRY(CopyIn(&g_state.stage_ids, ids_host, n * sizeof(int)));
   MoeTablePointers tables;
   GUFO_TRY(GroupDevLocked(static_cast<const int*>(g_state.stage_ids.ptr), tokens, k,
-                          experts, &tables));
+                          experts, false, &tables));
   gufo::MoeTables header;
   GUFO_TRY(CopyOut(&header, tables.header, sizeof header));
   if (header.n_invalid != 0) {

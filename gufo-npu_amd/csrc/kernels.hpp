@@ -95,6 +95,14 @@ hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int capacity
                           int* counts, int* offsets, int* pairs, uint8_t* pair_valid,
                           MoeSegment* segments, MoeTables* tables, hipStream_t stream);
 
+// The same pair_valid, segment list and *tables for a call of at most
+// kMaxSmallGroupPairs pairs, without the per-expert tables: what the expert kernels
+// read, in one wave.
+constexpr int kMaxSmallGroupPairs = 64;
+hipError_t LaunchMoeGroupSmall(const int* ids, int n_pairs, int experts, int capacity,
+                               uint8_t* pair_valid, MoeSegment* segments, MoeTables* tables,
+                               hipStream_t stream);
+
 // y[t][i] = sum over slots in order of weights[t*k+slot] * rows[(t*k+slot)][i],
 // accumulated in double; invalid pairs are skipped.
 hipError_t LaunchMoeCombine(const float* rows, const float* weights,

@@ -13,32 +13,58 @@ namespace {
 // probabilities), weights p/total/top with top = sum of the chosen p/total,
 // floored at the smallest normal fp16.
 //
-// One workgroup per token, one thread per expert.  Instead of k rounds of a
-// wave-wide arg-max, every thread counts the experts that precede its own in the
-// reference's order (higher probability, or equal probability and lower index):
-// that count is the expert's slot, and the experts whose count is below k are the
-// chosen ones.  The order is total, so the result does not depend on scheduling.
+// One workgroup per token, one thread per expert (four at 1024 experts).  Instead of k
+// rounds of a workgroup-wide arg-max, a thread counts the experts that precede its own
+// in the reference's order (higher probability, or equal probability and lower
+// index): that count is the expert's slot, and the experts whose count is below k are
+// the chosen ones.  The order is total, so the result does not depend on scheduling.
+//
+// Counting against every expert would be experts^2 comparisons, so it runs in two
+// levels.  First inside chunks of 64 experts: an expert preceded by k others of its own
+// chunk cannot be chosen.  The survivors (at most k per chunk) are listed, and each
+// counts its predecessors among the survivors only - which is its true count whenever
+// that is below k, because everything that precedes a chosen expert is itself chosen
+// and so survived its own chunk.
 
 constexpr int kRouteThreads = 256;
 constexpr int kRoutePerThread = kMaxRouteExperts / kRouteThreads;
+constexpr int kRouteChunk = 64;
+
+typedef double Double2 __attribute__((ext_vector_type(2)));
+
+// Whether expert `other_index` with probability `other` precedes (mine, my_index).
+__device__ __forceinline__ int Precedes(double other, int other_index, double mine, int my_index) {
+  return (other > mine || (other == mine && other_index < my_index)) ? 1 : 0;
+}
 
 __global__ __launch_bounds__(kRouteThreads) void RouteKernel(
     const float* __restrict__ logits, int experts, int k, int* ids, float* weights) {
-  __shared__ double lds_prob[kMaxRouteExperts];
+  __shared__ __align__(16) double lds_prob[kMaxRouteExperts];
+  __shared__ __align__(16) double lds_survivor[kMaxRouteExperts];
+  __shared__ int lds_survivor_index[kMaxRouteExperts];
   __shared__ double lds_chosen[kMaxRouteK];
   __shared__ double lds_wave[kRouteThreads / 64];
   __shared__ float lds_wave_max[kRouteThreads / 64];
+  __shared__ int lds_survivors;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const float* row = logits + static_cast<size_t>(blockIdx.x) * experts;
+  const int padded = (experts + kRouteChunk - 1) / kRouteChunk * kRouteChunk;
 
+  float logit[kRoutePerThread];
   float max_logit = -INFINITY;
-  for (int e = tid; e < experts; e += kRouteThreads) max_logit = fmaxf(max_logit, row[e]);
+#pragma unroll
+  for (int j = 0; j < kRoutePerThread; ++j) {
+    const int e = tid + kRouteThreads * j;
+    logit[j] = e < experts ? row[e] : -INFINITY;
+    max_logit = fmaxf(max_logit, logit[j]);
+  }
   for (int off = 32; off > 0; off >>= 1) {
     max_logit = fmaxf(max_logit, __shfl_xor(max_logit, off, 64));
   }
   if (lane == 0) lds_wave_max[wave] = max_logit;
+  if (tid == 0) lds_survivors = 0;
   __syncthreads();
   max_logit = fmaxf(fmaxf(lds_wave_max[0], lds_wave_max[1]),
                     fmaxf(lds_wave_max[2], lds_wave_max[3]));
@@ -50,9 +76,11 @@ __global__ __launch_bounds__(kRouteThreads) void RouteKernel(
     const int e = tid + kRouteThreads * j;
     prob[j] = 0.0;
     if (e < experts) {
-      prob[j] = exp(static_cast<double>(row[e]) - static_cast<double>(max_logit));
+      prob[j] = exp(static_cast<double>(logit[j]) - static_cast<double>(max_logit));
       lds_prob[e] = prob[j];
       total += prob[j];
+    } else if (e < padded) {
+      lds_prob[e] = -1.0;  // precedes nothing
     }
   }
   for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off, 64);
@@ -60,19 +88,52 @@ __global__ __launch_bounds__(kRouteThreads) void RouteKernel(
   __syncthreads();
   total = (lds_wave[0] + lds_wave[1]) + (lds_wave[2] + lds_wave[3]);
 
+  // Level one: predecessors inside the expert's own chunk of 64.
+  int mine_slot[kRoutePerThread];
 #pragma unroll
   for (int j = 0; j < kRoutePerThread; ++j) {
     const int e = tid + kRouteThreads * j;
+    mine_slot[j] = -1;
     if (e >= experts) continue;
-    const double mine = prob[j];
+    const int base = e & ~(kRouteChunk - 1);
+    const Double2* chunk = reinterpret_cast<const Double2*>(lds_prob + base);
     int before = 0;
-    for (int o = 0; o < experts; ++o) {
-      const double other = lds_prob[o];
-      before += (other > mine || (other == mine && o < e)) ? 1 : 0;
+#pragma unroll
+    for (int i = 0; i < kRouteChunk / 2; ++i) {
+      const Double2 others = chunk[i];
+      before += Precedes(others.x, base + 2 * i, prob[j], e);
+      before += Precedes(others.y, base + 2 * i + 1, prob[j], e);
+    }
+    if (before < k) {
+      mine_slot[j] = atomicAdd(&lds_survivors, 1);
+      lds_survivor[mine_slot[j]] = prob[j];
+      lds_survivor_index[mine_slot[j]] = e;
+    }
+  }
+  __syncthreads();
+
+  // Level two: predecessors among the survivors.
+  const int survivors = lds_survivors;
+#pragma unroll
+  for (int j = 0; j < kRoutePerThread; ++j) {
+    if (mine_slot[j] < 0) continue;
+    const int e = tid + kRouteThreads * j;
+    int before = 0;
+    int s = 0;
+    for (; s + 4 <= survivors; s += 4) {
+      const Double2 a = *reinterpret_cast<const Double2*>(lds_survivor + s);
+      const Double2 b = *reinterpret_cast<const Double2*>(lds_survivor + s + 2);
+      before += Precedes(a.x, lds_survivor_index[s], prob[j], e);
+      before += Precedes(a.y, lds_survivor_index[s + 1], prob[j], e);
+      before += Precedes(b.x, lds_survivor_index[s + 2], prob[j], e);
+      before += Precedes(b.y, lds_survivor_index[s + 3], prob[j], e);
+    }
+    for (; s < survivors; ++s) {
+      before += Precedes(lds_survivor[s], lds_survivor_index[s], prob[j], e);
     }
     if (before < k) {
       ids[static_cast<size_t>(blockIdx.x) * k + before] = e;
-      lds_chosen[before] = mine;
+      lds_chosen[before] = prob[j];
     }
   }
   __syncthreads();
@@ -208,6 +269,64 @@ __global__ __launch_bounds__(kGroupThreads) void MoeGroupKernel(
   }
 }
 
+// The segment list alone, for a call of at most 64 pairs (a decode step: a few tokens
+// times k), in one wave with no LDS: lane i owns pair i and learns, from the other
+// lanes' expert ids read lane by lane into scalar registers, how many earlier pairs
+// chose the same expert (its place in the expert's list), how many pairs did
+// altogether, and how many segments the lower-numbered experts take.  Segments come
+// out in ascending expert order with ascending pairs, as MoeGroupKernel writes them.
+__global__ __launch_bounds__(64) void MoeGroupSmallKernel(
+    const int* __restrict__ ids, int n_pairs, int experts, int capacity,
+    uint8_t* pair_valid, MoeSegment* segments, MoeTables* tables) {
+  const int lane = threadIdx.x;
+  const bool present = lane < n_pairs;
+  int expert = present ? ids[lane] : -1;
+  const bool valid = present && expert >= 0 && expert < experts;
+  if (!valid) expert = -1;
+  if (present) pair_valid[lane] = valid ? 1 : 0;
+
+  int place = 0;  // earlier pairs of the same expert
+  int count = 0;  // all pairs of the same expert
+  for (int j = 0; j < n_pairs; ++j) {
+    const int other = __builtin_amdgcn_readlane(expert, j);
+    const bool same = valid && other == expert;
+    place += (same && j < lane) ? 1 : 0;
+    count += same ? 1 : 0;
+  }
+  const bool leads = valid && place == 0;
+  const int own_segments = leads ? (count + capacity - 1) / capacity : 0;
+  int first_segment = 0;   // segments of lower-numbered experts
+  int total_segments = 0;
+  int distinct = 0;
+  for (int j = 0; j < n_pairs; ++j) {
+    const int other_segments = __builtin_amdgcn_readlane(own_segments, j);
+    if (other_segments == 0) continue;  // uniform
+    const int other = __builtin_amdgcn_readlane(expert, j);
+    first_segment += (valid && other < expert) ? other_segments : 0;
+    total_segments += other_segments;
+    ++distinct;
+  }
+  if (valid) {
+    const int segment = first_segment + place / capacity;
+    const int slot = place - (place / capacity) * capacity;
+    segments[segment].pair[slot] = lane;
+    if (slot == 0) {
+      const int here = min(capacity, count - place);
+      segments[segment].expert = expert;
+      segments[segment].n_pairs = here;
+      // Unused entries repeat a pair of the segment, so that reading them is harmless.
+      for (int f = here; f < kMaxGemvTokens; ++f) segments[segment].pair[f] = lane;
+    }
+  }
+  const int invalid = __builtin_popcountll(__ballot(present && !valid));
+  if (lane == 0) {
+    tables->n_segments = total_segments;
+    tables->n_distinct = distinct;
+    tables->n_invalid = invalid;
+    tables->pad = 0;
+  }
+}
+
 // ---- combine -----------------------------------------------------------------
 // out[t][i] = sum over slots in slot order of weight * routed row, in double
 // (src/models/qwen35/reference.cpp:595-606 of the reference).  One fixed order,
@@ -251,6 +370,18 @@ hipError_t LaunchMoeGroup(const int* ids, int n_pairs, int experts, int capacity
   hipLaunchKernelGGL(MoeGroupKernel, dim3(1), dim3(kGroupThreads), 0, stream, ids,
                      n_pairs, experts, capacity, counts, offsets, pairs, pair_valid,
                      segments, tables);
+  return hipGetLastError();
+}
+
+hipError_t LaunchMoeGroupSmall(const int* ids, int n_pairs, int experts, int capacity,
+                               uint8_t* pair_valid, MoeSegment* segments, MoeTables* tables,
+                               hipStream_t stream) {
+  if (n_pairs < 0 || n_pairs > kMaxSmallGroupPairs || experts < 1 || capacity < 1 ||
+      capacity > kMaxGemvTokens) {
+    return hipErrorInvalidValue;
+  }
+  hipLaunchKernelGGL(MoeGroupSmallKernel, dim3(1), dim3(64), 0, stream, ids, n_pairs, experts,
+                     capacity, pair_valid, segments, tables);
   return hipGetLastError();
 }
 
