@@ -49,7 +49,25 @@ def parse_args():
                     help="for a `rocprofv3 --pmc` run: a few plain launches of every decode "
                          "stage plus the read and write probes (known byte counts that "
                          "calibrate the memory counters), no timing")
+    ap.add_argument("--prefill-counters", action="store_true",
+                    help="for a `rocprofv3` run: a few plain launches of the prefill GEMM "
+                         "(config 5), no timing")
     return ap.parse_args()
+
+
+def run_prefill_counters(capi, cfg, synth, launches=6):
+    """Plain launches of the config-5 GEMM for a trace or counter run."""
+    spec = cfg.CONFIG5
+    mw = capi.Matrix(spec.ggml_type, spec.build(), spec.rows, spec.cols)
+    a_bits = synth.bf16_round(synth.activations(cfg.CONFIG5_TOKENS, spec.cols, cfg.CONFIG5_A_SEED))
+    da = capi.DeviceBuffer.from_array(a_bits)
+    dc = capi.DeviceBuffer(4 * cfg.CONFIG5_TOKENS * spec.rows)
+    for _ in range(launches):
+        capi.gemm_q4k_bf16_dev(mw, da, cfg.CONFIG5_TOKENS, dc)
+        capi.synchronize()
+    print(json.dumps({"prefill_counters_run": {
+        "launches": launches, "tokens": cfg.CONFIG5_TOKENS, "rows": spec.rows, "cols": spec.cols,
+        "flops_per_launch": 2 * cfg.CONFIG5_TOKENS * spec.rows * spec.cols}}))
 
 
 def run_counters(capi, cfg, decode):
@@ -331,6 +349,9 @@ def main():
     capi.init(0)
     device, cus = capi.device_info()
     log(f"device: {device}, {cus} CUs")
+    if args.prefill_counters:
+        run_prefill_counters(capi, cfg, synth)
+        return
     t0 = time.perf_counter()
     decode = DecodeSet(capi, cfg, synth, args.layer_copies, args.lm_head_copies)
     log(f"weights resident: {args.layer_copies} layer copies, {args.lm_head_copies} "
