@@ -64,6 +64,25 @@ def test_gemm_unit_activations_return_the_weights(hip, oracle):
     m.destroy()
 
 
+def test_gemm_full_size_is_independent_of_token_order(hip):
+    # Config-5 size, every one of the 4096 x 6144 outputs: a token's row of C is computed
+    # from that token's activations alone, in an order that does not depend on where the
+    # token sits, so reversing the token order must reverse C bit for bit.  Any mix-up of
+    # tiles, stages of the LDS ring or store addresses breaks this.
+    say("gemm token order, full size")
+    spec = cfg.CONFIG5
+    w = spec.build()
+    bits, _ = bf16_activations(cfg.CONFIG5_TOKENS, spec.cols, cfg.CONFIG5_A_SEED)
+    m = hip.Matrix(spec.ggml_type, w, spec.rows, spec.cols)
+    forward = hip.gemm_q4k_bf16(m, bits)
+    backward = hip.gemm_q4k_bf16(m, np.ascontiguousarray(bits[::-1]))
+    assert bool(np.array_equal(forward.view(np.uint32), backward[::-1].view(np.uint32)))
+    # and a second run repeats the first
+    again = hip.gemm_q4k_bf16(m, bits)
+    assert bool(np.array_equal(forward.view(np.uint32), again.view(np.uint32)))
+    m.destroy()
+
+
 def test_gemm_rejects_other_types(hip):
     say("gemm type check")
     w = synth.kquant_matrix(synth.Q6_K, 32, 256, 1)

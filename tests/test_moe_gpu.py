@@ -123,6 +123,19 @@ def test_moe_ffn_small_with_crowded_experts(hip, oracle):
         single = hip.moe_ffn(mg, mu, md, experts, x[t:t + 1], ids[t:t + 1], weights[t:t + 1])
         assert same(single[0], y[t])
     assert same(y, hip.moe_ffn(mg, mu, md, experts, x, ids, weights))
+    # a caller may name an expert twice in one token: both slots count, in slot order
+    twice = ids.copy()
+    twice[:, 1] = twice[:, 0]
+    y_twice = hip.moe_ffn(mg, mu, md, experts, x, twice, weights)
+    total = np.zeros(y_twice.shape, np.float64)
+    for slots in ((0,), (1,), (2, 3)):  # the output is linear in the slot weights
+        part = np.zeros_like(weights)
+        part[:, slots] = weights[:, slots]
+        total += hip.moe_ffn(mg, mu, md, experts, x, twice, part)
+    assert oracle.rel_l2(y_twice, total) <= 1e-6
+    for t in (0, tokens - 1):
+        single = hip.moe_ffn(mg, mu, md, experts, x[t:t + 1], twice[t:t + 1], weights[t:t + 1])
+        assert same(single[0], y_twice[t])
     with pytest.raises(hip.LogicError):
         bad = ids.copy()
         bad[0, 0] = experts
