@@ -218,6 +218,19 @@ def run_details(capi, cfg, synth, decode, args):
     for m in mats:
         m.destroy()
 
+    log("other row types of real files (not in the configurations), N=1, 40 copies from HBM:")
+    for name, ggml_type, rows, cols in (("q8_0 2048x2048", synth.Q8_0, 2048, 2048),
+                                        ("f32 router 257x2048", synth.F32, 257, 2048)):
+        host = synth.matrix(ggml_type, rows, cols, 7)
+        mats = [capi.Matrix(ggml_type, host, rows, cols) for _ in range(40)]
+        y2 = capi.DeviceBuffer(4 * rows)
+        ms = time_recorded(capi, [lambda m=m: capi.gemv_dev([capi.whole(m)], x, 1, y2)
+                                  for m in mats])
+        report(name, host.size, ms)
+        for m in mats:
+            m.destroy()
+        y2.free()
+
     log("config 3, MTP-verify FFN (gate|up 9216x2560 Q4_K, down 2560x9216 Q6_K), 8 copies:")
     gate, up, down = (cfg.CONFIG3[n] for n in ("gate", "up", "down"))
     hg, hu, hd = gate.build(), up.build(), down.build()

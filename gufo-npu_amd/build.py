@@ -11,8 +11,8 @@ CSRC = PACKAGE_DIR / "csrc"
 HOST = PACKAGE_DIR / "host"
 LIB_DIR = PACKAGE_DIR / "lib"
 
-HIP_SOURCES = ["capi.hip", "kquant_gemv.hip", "kquant_gemm_mfma.hip", "moe.hip",
-               "aux_kernels.hip"]
+HIP_SOURCES = ["capi.hip", "kquant_gemv.hip", "f32_gemv.hip", "kquant_gemm_mfma.hip",
+               "moe.hip", "aux_kernels.hip"]
 # -packed-fp32-ops off: no v_pk_*_f32 is generated.  -ffp-contract=off: fused
 # multiply-adds happen only where the source writes them, so the arithmetic of a
 # token column is the same in every kernel instantiation.

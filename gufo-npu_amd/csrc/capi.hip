@@ -346,6 +346,13 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                 experts);
   }
   const size_t ffn = gate->rows / e;
+  for (const gufo_hip_matrix* m : {gate, up, down}) {
+    if (m->type != GUFO_HIP_Q4_K && m->type != GUFO_HIP_Q5_K && m->type != GUFO_HIP_Q6_K) {
+      return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                  "expert tensors must be Q4_K, Q5_K or Q6_K; this one has ggml type %d",
+                  m->type);
+    }
+  }
   if (tokens == 0) return GUFO_HIP_OK;
   if (x == nullptr || y == nullptr || ids == nullptr || weights == nullptr) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: null buffer");
@@ -519,13 +526,13 @@ int gufo_hip_device_info(char* name, size_t name_bytes, int* compute_units) {
 }
 
 size_t gufo_hip_block_bytes(int ggml_type) {
-  return static_cast<size_t>(gufo::BlockBytes(ggml_type));
+  return static_cast<size_t>(gufo::FormatBlockBytes(ggml_type));
 }
 
 size_t gufo_hip_row_bytes(int ggml_type, size_t cols) {
-  const size_t block = gufo_hip_block_bytes(ggml_type);
-  if (block == 0 || cols % gufo::kSuperBlock != 0) return 0;
-  return cols / gufo::kSuperBlock * block;
+  const size_t per_super_block = static_cast<size_t>(gufo::BlockBytes(ggml_type));
+  if (per_super_block == 0 || cols % gufo::kSuperBlock != 0) return 0;
+  return cols / gufo::kSuperBlock * per_super_block;
 }
 
 int gufo_hip_malloc(void** device_ptr, size_t bytes) {
@@ -581,7 +588,9 @@ int gufo_hip_matrix_create(int ggml_type, const void* host_blocks, size_t rows,
   const size_t row_bytes = gufo_hip_row_bytes(ggml_type, cols);
   if (row_bytes == 0) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
-                "row is not a whole number of blocks (%zu values)", cols);
+                "row is not a whole number of blocks (%zu values; this backend takes rows "
+                "of a multiple of 256 values for every type)",
+                cols);
   }
   if (rows > 0xFFFFFFF0ull || cols > (1ull << 24)) {
     return Fail(GUFO_HIP_ERR_SHAPE, "matrix %zu x %zu exceeds the launch limits", rows, cols);

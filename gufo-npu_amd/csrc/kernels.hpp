@@ -42,6 +42,10 @@ int GemvMaxTokens(int type, uint32_t blocks_per_row);
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream);
 
+// The same for rows stored as fp32 (LaunchGemv forwards type 0 here).
+hipError_t LaunchGemvF32(const GemvLaunch& launch, const float* x, int tokens, float* y,
+                         hipStream_t stream);
+
 // ---- mixture of experts ------------------------------------------------------
 
 // One routed expert and up to four of the (token, slot) pairs that chose it.

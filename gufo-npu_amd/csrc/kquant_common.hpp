@@ -5,6 +5,10 @@
 //   Q4_K 144 B: d, dmin (fp16) | 12 packed scale bytes | qs[128]
 //   Q5_K 176 B: d, dmin (fp16) | 12 packed scale bytes | qh[32] | qs[128]
 //   Q6_K 210 B: ql[128] | qh[64] | int8 scales[16] | d (fp16)
+//   Q8_0  34 B: d (fp16) | 32 int8          (src/core/quant.cpp:22-31), 32 values
+//   F32    4 B: the value
+// The kernels walk every row in steps of 256 values - one K-quant super-block, eight
+// Q8_0 blocks or 256 floats - so every row length is a multiple of 256.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -12,13 +16,30 @@
 
 namespace gufo {
 
+constexpr int kTypeF32 = 0;
+constexpr int kTypeQ80 = 8;
 constexpr int kTypeQ4K = 12;
 constexpr int kTypeQ5K = 13;
 constexpr int kTypeQ6K = 14;
 constexpr int kSuperBlock = 256;
 
+// Bytes of 256 consecutive values of a row; 0 for a type the kernels do not take.
 __host__ __device__ constexpr int BlockBytes(int type) {
-  return type == kTypeQ4K ? 144 : type == kTypeQ5K ? 176 : type == kTypeQ6K ? 210 : 0;
+  return type == kTypeQ4K   ? 144
+         : type == kTypeQ5K ? 176
+         : type == kTypeQ6K ? 210
+         : type == kTypeQ80 ? 8 * 34
+         : type == kTypeF32 ? 256 * 4
+                            : 0;
+}
+
+// Bytes and values of one block as the GGUF format defines it
+// (src/core/quant.cpp:186-219 of the reference).
+__host__ __device__ constexpr int FormatBlockBytes(int type) {
+  return type == kTypeQ80 ? 34 : type == kTypeF32 ? 4 : BlockBytes(type);
+}
+__host__ __device__ constexpr int FormatBlockValues(int type) {
+  return type == kTypeQ80 ? 32 : type == kTypeF32 ? 1 : BlockBytes(type) != 0 ? 256 : 0;
 }
 
 // fp16 bits -> fp32, exact for every input (subnormals included): the hardware

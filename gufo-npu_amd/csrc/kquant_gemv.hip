@@ -503,9 +503,60 @@ struct RawQ6 {
   }
 };
 
+// Q8_0.  256 values are eight blocks of 34 bytes (fp16 scale, 32 int8).  Lane p owns
+// blocks 2p and 2p+1 - values 64p .. 64p+63, the split Q4_K's sub-blocks 2p, 2p+1 have,
+// so the activation layout is XK4's - at bytes 68p .. 68p+67 of the 272.  The int8
+// weights are dot4 operands as they are.  |sum of 32 q*X| can pass 2^31, so the three
+// limbs are summed apart (each below 2^19) and joined in fp32.
+struct RawQ8 {
+  U32x4 q[2][2];
+  uint32_t d[2];
+
+  __device__ __forceinline__ void Load(const uint8_t* blk, int lane4) {
+    const uint8_t* mine = blk + 68 * lane4;
+    d[0] = Load2(mine);
+    q[0][0] = Load16Align2(mine + 2);
+    q[0][1] = Load16Align2(mine + 18);
+    d[1] = Load2(mine + 34);
+    q[1][0] = Load16Align2(mine + 36);
+    q[1][1] = Load16Align2(mine + 52);
+  }
+
+  __device__ __forceinline__ static float BlockDot(const U32x4 (&codes)[2],
+                                                   const uint32_t (&limb)[3][8]) {
+    float joined = 0.0f;
+#pragma unroll
+    for (int l = 2; l >= 0; --l) {
+      int acc = 0;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) acc = Dot4(codes[w >> 2][w & 3], limb[l][w], acc);
+      joined = Fma(joined, 256.0f, static_cast<float>(acc));
+    }
+    return joined;
+  }
+
+  template <int NTOK, typename XSource>
+  __device__ __forceinline__ void Mac(int /*lane4*/, const XSource& source,
+                                      float (&acc)[NTOK]) const {
+    const float scale0 = HalfBitsToFloat(d[0]);
+    const float scale1 = HalfBitsToFloat(d[1]);
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+      const XK4 x = source.Get(t);
+      float part = scale0 * (BlockDot(q[0], x.limb[0]) * x.xs[0]);
+      part = Fma(scale1, BlockDot(q[1], x.limb[1]) * x.xs[1], part);
+      acc[t] += part;
+    }
+  }
+};
+
 template <int TYPE>
 struct RawOf {
   using Type = RawK4<TYPE == kTypeQ5K>;
+};
+template <>
+struct RawOf<kTypeQ80> {
+  using Type = RawQ8;
 };
 template <>
 struct RawOf<kTypeQ6K> {
@@ -856,6 +907,7 @@ void SetGemvComputeUnits(int compute_units) {
 int DeviceComputeUnits() { return g_compute_units; }
 
 int GemvMaxTokens(int type, uint32_t blocks_per_row) {
+  if (type == kTypeF32) return kMaxGemvTokens;  // no staging in LDS
   const size_t per_token = LdsBytes(type, blocks_per_row, 1);
   if (per_token == 0) return 0;
   const size_t fit = kGemvMaxLdsBytes / per_token;
@@ -864,6 +916,7 @@ int GemvMaxTokens(int type, uint32_t blocks_per_row) {
 
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream) {
+  if (type == kTypeF32) return LaunchGemvF32(launch, x, tokens, y, stream);
   if (!ValidLaunch(type, launch) || tokens < 1 ||
       tokens > GemvMaxTokens(type, launch.blocks_per_row)) {
     return hipErrorInvalidValue;
@@ -881,13 +934,17 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
   switch (type) {
     case kTypeQ4K: return LaunchTyped<kTypeQ4K>(prm, x, tokens, y, grid, lds_bytes, stream);
     case kTypeQ5K: return LaunchTyped<kTypeQ5K>(prm, x, tokens, y, grid, lds_bytes, stream);
-    default: return LaunchTyped<kTypeQ6K>(prm, x, tokens, y, grid, lds_bytes, stream);
+    case kTypeQ6K: return LaunchTyped<kTypeQ6K>(prm, x, tokens, y, grid, lds_bytes, stream);
+    case kTypeQ80: return LaunchTyped<kTypeQ80>(prm, x, tokens, y, grid, lds_bytes, stream);
+    default: return hipErrorInvalidValue;
   }
 }
 
 hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& moe,
                          bool swiglu, uint32_t max_segments, int max_pairs,
                          hipStream_t stream) {
+  // Expert tensors are K-quants (the reference's models hold them as Q4_K .. Q6_K).
+  if (type != kTypeQ4K && type != kTypeQ5K && type != kTypeQ6K) return hipErrorInvalidValue;
   if (!ValidLaunch(type, launch) || max_pairs < 1 ||
       GemvMaxTokens(type, launch.blocks_per_row) < kMaxGemvTokens) {
     return hipErrorInvalidValue;

@@ -57,7 +57,7 @@ public:
 // at the blocks as stored; it is read during construction only.
 struct Tensor {
   std::string name;
-  int ggml_type = 0;  // 12 = Q4_K, 13 = Q5_K, 14 = Q6_K
+  int ggml_type = 0;  // 0 = F32, 8 = Q8_0, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K
   std::vector<std::uint64_t> shape;
   const std::uint8_t* data = nullptr;
 };

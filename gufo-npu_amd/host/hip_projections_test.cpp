@@ -266,7 +266,7 @@ void RunDense(std::mt19937& rng) {
   Report("partial block throws std::invalid_argument",
          Throws<std::invalid_argument>([&] { HipProjections p(bad); }));
   bad = model;
-  bad.layers[0].ffn_down[0].ggml_type = 8;
+  bad.layers[0].ffn_down[0].ggml_type = 1;  // F16: not a row type GgufProjections takes
   Report("unsupported type throws std::invalid_argument",
          Throws<std::invalid_argument>([&] { HipProjections p(bad); }));
 }

@@ -20,9 +20,9 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q5_K, Q6_K = 12, 13, 14
+F32, Q8_0, Q4_K, Q5_K, Q6_K = 0, 8, 12, 13, 14
 BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210}
-TYPE_NAMES = {Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
+TYPE_NAMES = {F32: "F32", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
 SUPER_BLOCK = 256
 # The reference's own test seed (tests/models/qwen35/gguf_dot_test.cpp:91).
 BASE_SEED = 20261105
@@ -58,6 +58,33 @@ def kquant_matrix(ggml_type: int, rows: int, cols: int, seed: int) -> np.ndarray
     else:
         data[:, 208:210] = _half_scales(gen, n_blocks)
     return data.reshape(rows, -1)
+
+
+def q8_0_matrix(rows: int, cols: int, seed: int) -> np.ndarray:
+    """rows x (cols/32*34) uint8 of Q8_0 blocks: d = fp16(|N(0, 0.02)|), 32 uniform int8
+    (how the reference's own test builds such rows, tests/models/qwen35/gguf_dot_test.cpp:61-70)."""
+    if cols % 32 != 0:
+        raise ValueError("row is not a whole number of blocks")
+    n_blocks = rows * (cols // 32)
+    gen = rng(seed)
+    data = gen.integers(0, 256, size=(n_blocks, 34), dtype=np.uint8)
+    data[:, 0:2] = _half_scales(gen, n_blocks)
+    return data.reshape(rows, -1)
+
+
+def f32_matrix(rows: int, cols: int, seed: int) -> np.ndarray:
+    """rows x (cols*4) uint8: fp32 N(0, 0.05) weights as a file stores them."""
+    w = rng(seed).standard_normal((rows, cols), dtype=np.float32) * np.float32(0.05)
+    return np.ascontiguousarray(w).view(np.uint8).reshape(rows, cols * 4)
+
+
+def matrix(ggml_type: int, rows: int, cols: int, seed: int) -> np.ndarray:
+    """A synthetic matrix of any row type the backend takes."""
+    if ggml_type == F32:
+        return f32_matrix(rows, cols, seed)
+    if ggml_type == Q8_0:
+        return q8_0_matrix(rows, cols, seed)
+    return kquant_matrix(ggml_type, rows, cols, seed)
 
 
 def activations(tokens: int, cols: int, seed: int) -> np.ndarray:

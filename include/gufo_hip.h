@@ -34,8 +34,13 @@
 extern "C" {
 #endif
 
-/* ggml tensor type ids, numerically as in GGUF (src/core/gguf.hpp:16-24). */
+/* ggml tensor type ids, numerically as in GGUF (src/core/gguf.hpp:16-24): the five
+ * row types GgufProjections multiplies (gguf_projections.cpp:58-75).  F32 and Q8_0
+ * rows (routers, gates, a few projections of real files) go through the dense
+ * products only; expert tensors and the prefill GEMM take K-quants. */
 enum gufo_hip_type {
+  GUFO_HIP_F32 = 0,
+  GUFO_HIP_Q8_0 = 8,
   GUFO_HIP_Q4_K = 12,
   GUFO_HIP_Q5_K = 13,
   GUFO_HIP_Q6_K = 14
@@ -85,10 +90,14 @@ int gufo_hip_device_info(char* name, size_t name_bytes, int* compute_units);
 
 /* ---- block geometry: quant::BlockBytes / RowBytes (src/core/quant.cpp:202-227) */
 
-/* Bytes per 256-value super-block; 0 for a type this backend does not take. */
+/* Bytes of one block of the format (144 / 176 / 210 for the 256-value K-quant
+ * super-blocks, 34 for Q8_0's 32 values, 4 for F32); 0 for a type this backend does
+ * not take. */
 size_t gufo_hip_block_bytes(int ggml_type);
-/* Bytes of a row of `cols` values; 0 when cols is not a whole number of blocks
- * (where RowBytes throws std::invalid_argument). */
+/* Bytes of a row of `cols` values; 0 when cols is not a multiple of 256 (where
+ * RowBytes throws std::invalid_argument for a partial block).  This backend walks
+ * every row in steps of 256 values, so Q8_0 and F32 rows must be a multiple of 256
+ * long too, which is stricter than the reference's 32 and 1. */
 size_t gufo_hip_row_bytes(int ggml_type, size_t cols);
 
 /* ---- device memory for callers that keep x / y resident ------------------- */

@@ -52,14 +52,28 @@ size_t gufo_oracle_block_bytes(int type) {
     case GUFO_ORACLE_Q4_K: return 144; /* 2+2+12+128 */
     case GUFO_ORACLE_Q5_K: return 176; /* 2+2+12+32+128 */
     case GUFO_ORACLE_Q6_K: return 210; /* 128+64+16+2 */
+    case GUFO_ORACLE_Q8_0: return 34;  /* 2+32 */
+    case GUFO_ORACLE_F32: return 4;
+    default: return 0;
+  }
+}
+
+size_t gufo_oracle_block_elements(int type) {
+  switch (type) {
+    case GUFO_ORACLE_Q4_K:
+    case GUFO_ORACLE_Q5_K:
+    case GUFO_ORACLE_Q6_K: return kSuper;
+    case GUFO_ORACLE_Q8_0: return kSub;
+    case GUFO_ORACLE_F32: return 1;
     default: return 0;
   }
 }
 
 size_t gufo_oracle_row_bytes(int type, size_t n) {
   const size_t bytes = gufo_oracle_block_bytes(type);
-  if (bytes == 0 || n % kSuper != 0) return 0;
-  return n / kSuper * bytes;
+  const size_t elements = gufo_oracle_block_elements(type);
+  if (bytes == 0 || n % elements != 0) return 0;
+  return n / elements * bytes;
 }
 
 /* core/quant.cpp:158-167.  Twelve bytes hold eight 6-bit scales and eight 6-bit
@@ -138,8 +152,25 @@ static void dequant_q6(const uint8_t* src, float* dst, size_t blocks) {
   }
 }
 
+/* core/quant.cpp:22-31: fp16 scale times 32 int8. */
+static void dequant_q8_0(const uint8_t* src, float* dst, size_t blocks) {
+  for (size_t b = 0; b < blocks; ++b, src += 34, dst += kSub) {
+    const float d = gufo_oracle_half_to_float(load_u16(src));
+    const int8_t* q = (const int8_t*)(src + 2);
+    for (int j = 0; j < kSub; ++j) dst[j] = d * (float)q[j];
+  }
+}
+
 int gufo_oracle_dequantize(int type, const uint8_t* src, float* dst, size_t n) {
-  if (gufo_oracle_block_bytes(type) == 0 || n % kSuper != 0) return -1;
+  if (gufo_oracle_row_bytes(type, n) == 0 && n != 0) return -1;
+  if (type == GUFO_ORACLE_F32) {
+    memcpy(dst, src, n * sizeof(float));
+    return 0;
+  }
+  if (type == GUFO_ORACLE_Q8_0) {
+    dequant_q8_0(src, dst, n / kSub);
+    return 0;
+  }
   const size_t blocks = n / kSuper;
   switch (type) {
     case GUFO_ORACLE_Q4_K: dequant_k4(src, dst, blocks, 0); return 0;
@@ -207,6 +238,40 @@ float gufo_oracle_dot_q6_k(const uint8_t* row, const float* x, size_t n) {
   return total;
 }
 
+/* models/qwen35/gguf_dot.hpp:62-74: per block an fp32 sum of q*x in order, times the
+ * block's scale into the row sum. */
+float gufo_oracle_dot_q8_0(const uint8_t* row, const float* x, size_t n) {
+  float sum = 0.0f;
+  for (size_t b = 0; b < n / kSub; ++b, row += 34) {
+    const int8_t* q = (const int8_t*)(row + 2);
+    float block = 0.0f;
+    for (int j = 0; j < kSub; ++j) block += (float)q[j] * x[b * kSub + j];
+    sum += gufo_oracle_half_to_float(load_u16(row)) * block;
+  }
+  return sum;
+}
+
+/* core/vec.hpp:36-51: eight interleaved partial sums, added in order, then the tail. */
+float gufo_oracle_dot_f32(const uint8_t* row, const float* x, size_t n) {
+  float lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  size_t i = 0;
+  for (; i + 8 <= n; i += 8) {
+    for (int l = 0; l < 8; ++l) {
+      float w;
+      memcpy(&w, row + 4 * (i + (size_t)l), sizeof w);
+      lanes[l] += w * x[i + (size_t)l];
+    }
+  }
+  float total = 0.0f;
+  for (int l = 0; l < 8; ++l) total += lanes[l];
+  for (; i < n; ++i) {
+    float w;
+    memcpy(&w, row + 4 * i, sizeof w);
+    total += w * x[i];
+  }
+  return total;
+}
+
 static double dot_double_buf(int type, const uint8_t* row, const float* x,
                              size_t n, float* w) {
   gufo_oracle_dequantize(type, row, w, n);
@@ -228,6 +293,8 @@ static float dot_fused(int type, const uint8_t* row, const float* x, size_t n) {
   switch (type) {
     case GUFO_ORACLE_Q4_K: return dot_k4(row, x, n, 0);
     case GUFO_ORACLE_Q5_K: return dot_k4(row, x, n, 1);
+    case GUFO_ORACLE_Q8_0: return gufo_oracle_dot_q8_0(row, x, n);
+    case GUFO_ORACLE_F32: return gufo_oracle_dot_f32(row, x, n);
     default: return gufo_oracle_dot_q6_k(row, x, n);
   }
 }
@@ -299,13 +366,13 @@ int gufo_oracle_matmul(int n_parts, const uint8_t* const* data, const int* types
                        const size_t* first, const size_t* rows, size_t in,
                        const float* x, int tokens, float* y, int precision,
                        int threads) {
-  if (n_parts <= 0 || tokens < 0 || in == 0 || in % kSuper != 0) return -1;
+  if (n_parts <= 0 || tokens < 0 || in == 0) return -1;
   size_t* first_job = (size_t*)malloc(((size_t)n_parts + 1) * sizeof(size_t));
   MatMulTask task;
   memset(&task, 0, sizeof task);
   first_job[0] = 0;
   for (int p = 0; p < n_parts; ++p) {
-    if (gufo_oracle_block_bytes(types[p]) == 0) {
+    if (gufo_oracle_row_bytes(types[p], in) == 0) { /* unknown type or partial block */
       free(first_job);
       return -1;
     }

@@ -11,10 +11,12 @@
  * formula, fixes its output):
  *   half_to_float      fp16 known-answer table of tests/core/quant_test.cpp:51-70,
  *                      exhaustive comparison of all 65,536 inputs with numpy float16
- *   dequantize         bit-exact against the gguf-py fixtures Q4_K/Q5_K/Q6_K.{bin,f32}
- *                      (tests/fixtures/quant) and against the compiled reference
+ *   dequantize         bit-exact against the gguf-py fixtures Q4_K/Q5_K/Q6_K/Q8_0
+ *                      .{bin,f32} (tests/fixtures/quant) and against the compiled
+ *                      reference; F32 is a copy
  *   scale_min_k4       round trip through the packer's inverse over all 64x64 values
- *   dot_q4_k/q5_k/q6_k closed form: dequantize + double sum, limit 2e-5 of sum|w x|
+ *   dot_q4_k/q5_k/q6_k, dot_q8_0, dot_f32
+ *                      closed form: dequantize + double sum, limit 2e-5 of sum|w x|
  *                      (tests/models/qwen35/gguf_dot_test.cpp:116); compiled reference
  *   matmul             "each output is one dot product": equality with single dots at
  *                      the documented index t*stride+offset+r; compiled reference
@@ -34,13 +36,21 @@ extern "C" {
 #endif
 
 /* ggml type ids (core/gguf.hpp:16-24). */
-enum { GUFO_ORACLE_Q4_K = 12, GUFO_ORACLE_Q5_K = 13, GUFO_ORACLE_Q6_K = 14 };
+enum {
+  GUFO_ORACLE_F32 = 0,
+  GUFO_ORACLE_Q8_0 = 8,
+  GUFO_ORACLE_Q4_K = 12,
+  GUFO_ORACLE_Q5_K = 13,
+  GUFO_ORACLE_Q6_K = 14
+};
 
 /* core/quant.cpp:129-155 */
 float gufo_oracle_half_to_float(uint16_t h);
 /* core/quant.cpp:202-219; 0 for a type this path does not cover */
 size_t gufo_oracle_block_bytes(int type);
-/* core/quant.cpp:221-227; 0 when n is not a whole number of 256-value blocks */
+/* core/quant.cpp:186-200; 0 for a type this path does not cover */
+size_t gufo_oracle_block_elements(int type);
+/* core/quant.cpp:221-227; 0 when n is not a whole number of blocks */
 size_t gufo_oracle_row_bytes(int type, size_t n);
 /* core/quant.cpp:158-167 */
 void gufo_oracle_scale_min_k4(size_t j, const uint8_t* packed, uint8_t* scale,
@@ -54,6 +64,11 @@ float gufo_oracle_dot_q4_k(const uint8_t* row, const float* x, size_t n);
 float gufo_oracle_dot_q5_k(const uint8_t* row, const float* x, size_t n);
 /* models/qwen35/gguf_dot.hpp:260-289 (portable body of DotQ6_K) */
 float gufo_oracle_dot_q6_k(const uint8_t* row, const float* x, size_t n);
+/* models/qwen35/gguf_dot.hpp:62-74 (portable body of DotQ8_0) */
+float gufo_oracle_dot_q8_0(const uint8_t* row, const float* x, size_t n);
+/* core/vec.hpp:36-51 (portable body of vec::Dot, which DotF32 calls,
+ * models/qwen35/gguf_dot.hpp:71-75) */
+float gufo_oracle_dot_f32(const uint8_t* row, const float* x, size_t n);
 /* dequantize then sum in double: GgufProjections' kDouble path,
  * models/qwen35/gguf_projections.cpp:48-54,277-282 */
 double gufo_oracle_dot_double(int type, const uint8_t* row, const float* x,

@@ -16,7 +16,7 @@ ORACLE_DIR = Path(__file__).resolve().parent
 ORACLE_LIB = ORACLE_DIR / "libkquant_oracle.so"
 REF_LIB = ORACLE_DIR / "_ref" / "libgufo_ref.so"
 
-Q4_K, Q5_K, Q6_K = 12, 13, 14
+F32, Q8_0, Q4_K, Q5_K, Q6_K = 0, 8, 12, 13, 14
 _SZ = C.c_size_t
 _P = C.c_void_p
 
@@ -48,7 +48,7 @@ def lib() -> C.CDLL:
         o.gufo_oracle_scale_min_k4.argtypes = [_SZ, _P, _P, _P]
         o.gufo_oracle_dequantize.restype = C.c_int
         o.gufo_oracle_dequantize.argtypes = [C.c_int, _P, _P, _SZ]
-        for name in ("q4_k", "q5_k", "q6_k"):
+        for name in ("q4_k", "q5_k", "q6_k", "q8_0", "f32"):
             fn = getattr(o, f"gufo_oracle_dot_{name}")
             fn.restype = C.c_float
             fn.argtypes = [_P, _P, _SZ]
@@ -141,7 +141,7 @@ def dot(ggml_type: int, row: np.ndarray, x: np.ndarray, use_ref: bool = False) -
     row, x = _u8(row), _f32(x)
     if use_ref:
         return ref().ref_dot(ggml_type, _p(row), _p(x), x.size)
-    name = {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}[ggml_type]
+    name = {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k", Q8_0: "q8_0", F32: "f32"}[ggml_type]
     return getattr(lib(), f"gufo_oracle_dot_{name}")(_p(row), _p(x), x.size)
 
 

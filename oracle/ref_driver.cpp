@@ -45,6 +45,8 @@ RowDot DotFor(int type) {
     case GgmlType::kQ4_K: return &dot::DotQ4_K;
     case GgmlType::kQ5_K: return &dot::DotQ5_K;
     case GgmlType::kQ6_K: return &dot::DotQ6_K;
+    case GgmlType::kQ8_0: return &dot::DotQ8_0;
+    case GgmlType::kF32: return &dot::DotF32;
     default: return nullptr;
   }
 }

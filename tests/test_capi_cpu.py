@@ -25,7 +25,11 @@ def test_library_exports_every_declared_symbol():
 
 def test_block_geometry_without_device():
     assert [capi.block_bytes(t) for t in (12, 13, 14)] == [144, 176, 210]
-    assert capi.block_bytes(8) == 0 and capi.block_bytes(0) == 0
+    assert capi.block_bytes(synth.Q8_0) == 34 and capi.block_bytes(synth.F32) == 4
+    assert capi.block_bytes(1) == 0 and capi.block_bytes(30) == 0   # F16, BF16: not taken
+    assert capi.row_bytes(synth.Q8_0, 2048) == 2176
+    assert capi.row_bytes(synth.F32, 512) == 2048
+    assert capi.row_bytes(synth.Q8_0, 2016) == 0   # rows are multiples of 256 values here
     assert capi.row_bytes(synth.Q4_K, 2048) == 1152
     assert capi.row_bytes(synth.Q5_K, 512) == 352
     assert capi.row_bytes(synth.Q6_K, 6144) == 5040

@@ -13,7 +13,8 @@ from gufo_npu_amd import synth
 
 pytestmark = pytest.mark.gpu
 
-TYPES = [synth.Q4_K, synth.Q5_K, synth.Q6_K]
+TYPES = [synth.Q4_K, synth.Q5_K, synth.Q6_K]     # the formats that have a fixture pair
+ROW_TYPES = TYPES + [synth.Q8_0, synth.F32]      # every row type GgufProjections multiplies
 NAMES = synth.TYPE_NAMES
 TOLERANCE = 1e-4  # rel-L2, fp32 accumulation
 
@@ -28,7 +29,7 @@ def same_bits(a, b) -> bool:
                                np.ascontiguousarray(b).view(np.uint32)))
 
 
-@pytest.mark.parametrize("ggml_type", TYPES)
+@pytest.mark.parametrize("ggml_type", TYPES + [synth.Q8_0])
 def test_decode_matches_gguf_py_fixture_bit_for_bit(hip, ggml_type):
     # One row of the fixture's 512 values times the 512 unit vectors returns the
     # dequantized weights themselves: every code, scale and position is checked bit
@@ -55,11 +56,11 @@ SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("ggml_type", TYPES)
+@pytest.mark.parametrize("ggml_type", ROW_TYPES)
 @pytest.mark.parametrize("rows,cols", SHAPES)
 def test_gemv_parity(hip, oracle, ggml_type, rows, cols):
     seed = synth.BASE_SEED + ggml_type * 1000 + rows + cols
-    w = synth.kquant_matrix(ggml_type, rows, cols, seed)
+    w = synth.matrix(ggml_type, rows, cols, seed)
     m = hip.Matrix(ggml_type, w, rows, cols)
     for tokens in (1, 2, 3, 4):
         say("gemv", NAMES[ggml_type], rows, cols, "N", tokens)
@@ -101,6 +102,40 @@ def test_gemv_parts_row_ranges_and_mixed_types(hip, oracle):
             assert oracle.rel_l2(got[t, lo:hi], want[t, lo:hi]) <= TOLERANCE
     for m in (ma, mb, mc, md):
         m.destroy()
+
+
+def test_linear_in_style_stage_with_f32_and_q8_0_parts(hip, oracle):
+    # The linear-attention input stage of a real file: [qkv | z | alpha | beta] with the
+    # two small projections stored in fp32 and one matrix in Q8_0
+    # (Stage::kLinearIn, src/models/qwen35/projections.hpp:15-17 of the reference).
+    say("gemv mixed row types")
+    cols = 2048
+    specs = [(synth.Q5_K, 384), (synth.Q8_0, 256), (synth.F32, 16), (synth.F32, 16),
+             (synth.Q4_K, 64)]
+    blocks = [synth.matrix(t, rows, cols, 70 + i) for i, (t, rows) in enumerate(specs)]
+    mats = [hip.Matrix(t, b, rows, cols) for (t, rows), b in zip(specs, blocks)]
+    for tokens in (1, 3):
+        x = synth.activations(tokens, cols, 80 + tokens)
+        got = hip.gemv([hip.whole(m) for m in mats], x, tokens)
+        want = oracle.matmul([(t, b, 0, rows) for (t, rows), b in zip(specs, blocks)], x,
+                             precision="double")
+        assert got.shape == want.shape == (tokens, 736)
+        lo = 0
+        for (t, rows) in specs:
+            assert oracle.rel_l2(got[:, lo:lo + rows], want[:, lo:lo + rows]) <= TOLERANCE
+            lo += rows
+    for m in mats:
+        m.destroy()
+
+
+def test_f32_rows_return_themselves_for_unit_activations(hip):
+    say("f32 identity")
+    rows, cols = 9, 512
+    w = synth.f32_matrix(rows, cols, 91)
+    m = hip.Matrix(synth.F32, w, rows, cols)
+    y = hip.gemv([hip.whole(m)], np.eye(cols, dtype=np.float32), cols)
+    m.destroy()
+    assert same_bits(np.ascontiguousarray(y.T), w.view(np.float32).reshape(rows, cols))
 
 
 def test_gemv_many_tokens_and_empty(hip, oracle):
@@ -238,8 +273,10 @@ def test_error_codes(hip):
     w = synth.kquant_matrix(synth.Q4_K, 8, 512, 1)
     with pytest.raises(hip.InvalidArgumentError):  # partial block
         hip.Matrix(synth.Q4_K, w, 8, 500)
-    with pytest.raises(hip.InvalidArgumentError):  # unknown type (Q8_0 is not taken yet)
-        hip.Matrix(8, w, 8, 512)
+    with pytest.raises(hip.InvalidArgumentError):  # a type GgufProjections does not take: F16
+        hip.Matrix(1, w, 8, 512)
+    with pytest.raises(hip.InvalidArgumentError):  # Q8_0 rows are multiples of 256 values here
+        hip.Matrix(synth.Q8_0, synth.q8_0_matrix(4, 288, 1), 4, 288)
     a = hip.Matrix(synth.Q4_K, w, 8, 512)
     b = hip.Matrix(synth.Q4_K, synth.kquant_matrix(synth.Q4_K, 8, 256, 2), 8, 256)
     x = synth.activations(1, 512, 3)

@@ -37,7 +37,7 @@ def test_half_exhaustive_against_numpy(oracle):
 def test_block_geometry(oracle):
     lib = oracle.lib()
     assert [lib.gufo_oracle_block_bytes(t) for t in TYPES] == [144, 176, 210]
-    assert lib.gufo_oracle_block_bytes(8) == 0
+    assert lib.gufo_oracle_block_bytes(2) == 0
     assert lib.gufo_oracle_row_bytes(synth.Q6_K, 2048) == 1680
     assert lib.gufo_oracle_row_bytes(synth.Q4_K, 2000) == 0  # partial block
 
@@ -55,7 +55,7 @@ def test_dequantize_rejects_partial_block(oracle):
     with pytest.raises(ValueError):
         oracle.dequantize(synth.Q4_K, np.zeros(144, np.uint8), 255)
     with pytest.raises(ValueError):
-        oracle.dequantize(8, np.zeros(144, np.uint8), 256)
+        oracle.dequantize(2, np.zeros(144, np.uint8), 256)
 
 
 @pytest.mark.parametrize("ggml_type", TYPES)
@@ -139,6 +139,93 @@ def test_fused_dot_against_compiled_reference(ref_oracle, ggml_type):
             got = ref_oracle.dot(ggml_type, row, x)
             want = ref_oracle.dot(ggml_type, row, x, use_ref=True)
             assert abs(got - want) < 2e-5 * magnitude
+
+
+def q8_0_row(n, gen):
+    """Q8_0 blocks as the reference's gguf_dot_test.cpp:25-72 builds them: random int8,
+    fp16 scale normal, either sign, magnitude 2^-10..2^-1."""
+    blocks = n // 32
+    row = gen.integers(0, 256, size=(blocks, 34), dtype=np.uint8)
+    sign = gen.integers(0, 2, blocks).astype(np.uint16) << 15
+    exponent = (5 + gen.integers(0, 10, blocks)).astype(np.uint16) << 10
+    half = (sign | exponent | gen.integers(0, 1024, blocks).astype(np.uint16)).astype(np.uint16)
+    row[:, 0:2] = half.view(np.uint8).reshape(-1, 2)
+    return row.reshape(-1)
+
+
+def test_q8_0_and_f32_geometry(oracle):
+    lib = oracle.lib()
+    assert lib.gufo_oracle_block_bytes(synth.Q8_0) == 34
+    assert lib.gufo_oracle_block_bytes(synth.F32) == 4
+    assert lib.gufo_oracle_row_bytes(synth.Q8_0, 2048) == 2176
+    assert lib.gufo_oracle_row_bytes(synth.Q8_0, 2040) == 0   # partial block
+    assert lib.gufo_oracle_row_bytes(synth.F32, 7) == 28
+    assert lib.gufo_oracle_block_bytes(1) == 0                 # F16 is not on this path
+
+
+def test_q8_0_dequantize_matches_gguf_py_fixture_bit_for_bit(oracle):
+    raw = np.fromfile(GOLDEN / "quant" / "Q8_0.bin", dtype=np.uint8)
+    want = np.fromfile(GOLDEN / "quant" / "Q8_0.f32", dtype=np.float32)
+    assert raw.size == want.size // 32 * 34
+    got = oracle.dequantize(synth.Q8_0, raw, want.size)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q8_0_integer_special_case(oracle):
+    # d = 1: the row is the int8 codes themselves and the dot an integer dot product.
+    gen = synth.rng(5)
+    row = gen.integers(0, 256, size=(8, 34), dtype=np.uint8)
+    row[:, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    codes = row[:, 2:].reshape(-1).view(np.int8).astype(np.int64)
+    x = gen.integers(-8, 9, 256).astype(np.float32)
+    assert np.array_equal(oracle.dequantize(synth.Q8_0, row, 256), codes.astype(np.float32))
+    assert oracle.dot(synth.Q8_0, row, x) == float(np.dot(codes, x.astype(np.int64)))
+
+
+@pytest.mark.parametrize("n", [32, 256, 2048])
+def test_q8_0_and_f32_dots_against_double_sum(oracle, n):
+    gen = synth.rng(300 + n)
+    worst = 0.0
+    for _ in range(200):
+        row = q8_0_row(n, gen)
+        x = gen.standard_normal(n, dtype=np.float32)
+        w = oracle.dequantize(synth.Q8_0, row, n).astype(np.float64)
+        want, magnitude = float(np.dot(w, x.astype(np.float64))), float(np.sum(np.abs(w * x)))
+        worst = max(worst, abs(oracle.dot(synth.Q8_0, row, x) - want) / magnitude)
+        assert abs(oracle.dot_double(synth.Q8_0, row, x) - want) <= 1e-12 * magnitude
+        wf = gen.standard_normal(n + 3, dtype=np.float32)   # a tail after the 8-wide part
+        xf = gen.standard_normal(n + 3, dtype=np.float32)
+        want = float(np.dot(wf.astype(np.float64), xf.astype(np.float64)))
+        magnitude = float(np.sum(np.abs(wf.astype(np.float64) * xf)))
+        worst = max(worst, abs(oracle.dot(synth.F32, wf.view(np.uint8), xf) - want) / magnitude)
+        assert np.array_equal(oracle.dequantize(synth.F32, wf.view(np.uint8), n + 3), wf)
+    assert worst < 2e-5, worst
+
+
+def test_q8_0_and_f32_against_compiled_reference(ref_oracle):
+    gen = synth.rng(401)
+    for n in (256, 2048, 6144):
+        for _ in range(50):
+            row = q8_0_row(n, gen)
+            x = gen.standard_normal(n, dtype=np.float32)
+            got = ref_oracle.dequantize(synth.Q8_0, row, n)
+            assert np.array_equal(got, ref_oracle.dequantize(synth.Q8_0, row, n, use_ref=True))
+            magnitude = float(np.sum(np.abs(got.astype(np.float64) * x)))
+            assert abs(ref_oracle.dot(synth.Q8_0, row, x) -
+                       ref_oracle.dot(synth.Q8_0, row, x, use_ref=True)) < 2e-5 * magnitude
+            w = gen.standard_normal(n, dtype=np.float32)
+            magnitude = float(np.sum(np.abs(w.astype(np.float64) * x)))
+            assert abs(ref_oracle.dot(synth.F32, w.view(np.uint8), x) -
+                       ref_oracle.dot(synth.F32, w.view(np.uint8), x, use_ref=True)) \
+                < 2e-5 * magnitude
+    # the row loop over mixed parts, against the reference's pool
+    cols = 512
+    a, b = synth.q8_0_matrix(40, cols, 1), synth.f32_matrix(9, cols, 2)
+    x = synth.activations(3, cols, 3)
+    parts = [(synth.Q8_0, a, 3, 30), (synth.F32, b, 0, 9)]
+    got = ref_oracle.matmul(parts, x, threads=3)
+    want = ref_oracle.matmul(parts, x, threads=3, use_ref=True)
+    assert ref_oracle.rel_l2(got, want) < 1e-6
 
 
 def test_q4_k_integer_special_case(oracle):
