@@ -302,8 +302,8 @@ def run_details(capi, cfg, synth, decode, args):
         ms = time_recorded(capi, calls)
         mean_distinct = sum(distinct) / len(distinct)
         report(f"route+group+experts batch {tokens}", int(mean_distinct * per_expert), ms,
-               f"({mean_distinct:.1f} distinct experts; 5 kernels: "
-               f"route, group, gate|up, down, combine)")
+               f"({mean_distinct:.1f} distinct experts; kernels: route, "
+               f"{'' if tokens == 1 else 'group, '}gate|up, down, combine)")
         for b in keep:
             b.free()
     for m in (mg, mu, md):

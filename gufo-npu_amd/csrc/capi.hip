@@ -358,8 +358,15 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: null buffer");
   }
   if (!Aligned16(x)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
+  // One token: its slots are the segments, nothing to group (a kernel launch less per
+  // decode step); the combine fills the header from the ids instead.
+  const bool direct = tokens == 1;
   MoeTablePointers tables;
-  GUFO_TRY(GroupDevLocked(ids, tokens, k, experts, true, &tables));
+  if (direct) {
+    GUFO_TRY(ReserveMoeTables(k, experts, &tables));
+  } else {
+    GUFO_TRY(GroupDevLocked(ids, tokens, k, experts, true, &tables));
+  }
   const size_t n_pairs = static_cast<size_t>(tokens) * k;
   GUFO_TRY(Reserve(&g_state.moe_gate_up, n_pairs * 2 * ffn * sizeof(float)));
   GUFO_TRY(Reserve(&g_state.moe_out, n_pairs * hidden * sizeof(float)));
@@ -373,6 +380,8 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   args.tables = tables.header;
   args.segments = tables.segments;
   args.k = static_cast<uint32_t>(k);
+  args.direct_ids = direct ? ids : nullptr;
+  args.experts = experts;
 
   // [gate | up] of every pair: kExpertIn's layout.
   args.x = x;
@@ -420,8 +429,14 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                                      static_cast<uint32_t>(n_pairs), max_pairs,
                                      g_state.stream));
   }
-  GUFO_HIP_TRY(gufo::LaunchMoeCombine(routed, weights, tables.valid, tokens, k,
-                                      static_cast<int>(hidden), y, g_state.stream));
+  if (direct) {
+    GUFO_HIP_TRY(gufo::LaunchMoeCombineDirect(routed, weights, ids, experts, k,
+                                              static_cast<int>(hidden), y, tables.header,
+                                              g_state.stream));
+  } else {
+    GUFO_HIP_TRY(gufo::LaunchMoeCombine(routed, weights, tables.valid, tokens, k,
+                                        static_cast<int>(hidden), y, g_state.stream));
+  }
   g_state.moe_pending = true;
   return GUFO_HIP_OK;
 }

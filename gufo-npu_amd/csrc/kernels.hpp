@@ -72,6 +72,11 @@ struct MoeGemvArgs {
   float* y;             // output rows, one per pair, y_stride floats apart
   uint32_t k;           // slots per token
   size_t expert_bytes;  // bytes between experts, the same for every part of a launch
+  // One-token calls need no grouping: with direct_ids set, segment s is slot s alone,
+  // its expert direct_ids[s] (skipped when not below `experts`), and tables / segments
+  // are not read.
+  const int32_t* direct_ids;
+  int32_t experts;
 };
 
 // As LaunchGemv, once per segment: part p's rows start at
@@ -112,6 +117,13 @@ hipError_t LaunchMoeGroupSmall(const int* ids, int n_pairs, int experts, int cap
 hipError_t LaunchMoeCombine(const float* rows, const float* weights,
                             const uint8_t* pair_valid, int tokens, int k, int hidden,
                             float* y, hipStream_t stream);
+
+// The same for one token whose pairs were not grouped: a slot is valid when its id is
+// below `experts`; also fills *tables from the ids (what the grouping kernel would have
+// written), so that out-of-range ids are reported as after a grouped call.
+hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const int32_t* ids,
+                                  int experts, int k, int hidden, float* y, MoeTables* tables,
+                                  hipStream_t stream);
 
 // ---- prefill ------------------------------------------------------------------
 

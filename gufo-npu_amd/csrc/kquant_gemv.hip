@@ -801,8 +801,18 @@ __attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(kMaxTok)))) void KquantMoeGem
     const GemvParams prm, const MoeGemvArgs moe) {
   extern __shared__ __align__(16) U32x4 lds[];
   const uint32_t s = blockIdx.y;
-  if (s >= static_cast<uint32_t>(moe.tables->n_segments)) return;
-  const MoeSegment seg = moe.segments[s];
+  MoeSegment seg;
+  if (moe.direct_ids != nullptr) {
+    // An ungrouped one-token call: segment s is slot s.
+    seg.expert = moe.direct_ids[s];
+    if (seg.expert < 0 || seg.expert >= moe.experts) return;
+    seg.n_pairs = 1;
+#pragma unroll
+    for (int t = 0; t < kMaxGemvTokens; ++t) seg.pair[t] = static_cast<int32_t>(s);
+  } else {
+    if (s >= static_cast<uint32_t>(moe.tables->n_segments)) return;
+    seg = moe.segments[s];
+  }
   if (kMaxTok == 1 || seg.n_pairs == 1) {
     MoeSegmentBody<TYPE, 1, kSwiGlu>(prm, moe, seg, lds);
   } else if (kMaxTok >= 2 && seg.n_pairs == 2) {

@@ -346,7 +346,52 @@ __global__ __launch_bounds__(256) void MoeCombineKernel(
   y[static_cast<size_t>(t) * hidden + i] = static_cast<float>(acc);
 }
 
+// One token, pairs not grouped: validity comes from the ids themselves, and thread 0 of
+// the launch writes the header the grouping kernel would have written.
+__global__ __launch_bounds__(256) void MoeCombineDirectKernel(
+    const float* __restrict__ rows, const float* __restrict__ weights,
+    const int32_t* __restrict__ ids, int experts, int k, int hidden, float* __restrict__ y,
+    MoeTables* tables) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i == 0) {
+    int invalid = 0;
+    int distinct = 0;
+    for (int s = 0; s < k; ++s) {
+      const int e = ids[s];
+      if (e < 0 || e >= experts) {
+        ++invalid;
+        continue;
+      }
+      bool seen = false;
+      for (int r = 0; r < s; ++r) seen = seen || ids[r] == e;
+      distinct += seen ? 0 : 1;
+    }
+    tables->n_segments = k - invalid;
+    tables->n_distinct = distinct;
+    tables->n_invalid = invalid;
+    tables->pad = 0;
+  }
+  if (i >= hidden) return;
+  double acc = 0.0;
+  for (int slot = 0; slot < k; ++slot) {
+    const int e = ids[slot];
+    if (e < 0 || e >= experts) continue;
+    acc += static_cast<double>(weights[slot]) *
+           static_cast<double>(rows[static_cast<size_t>(slot) * hidden + i]);
+  }
+  y[i] = static_cast<float>(acc);
+}
+
 }  // namespace
+
+hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const int32_t* ids,
+                                  int experts, int k, int hidden, float* y, MoeTables* tables,
+                                  hipStream_t stream) {
+  if (hidden <= 0 || k <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(MoeCombineDirectKernel, dim3((hidden + 255) / 256), dim3(256), 0, stream,
+                     rows, weights, ids, experts, k, hidden, y, tables);
+  return hipGetLastError();
+}
 
 hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int* ids,
                        float* weights, hipStream_t stream) {
