@@ -72,14 +72,15 @@ __global__ __launch_bounds__(256) void ReadProbe(const U32x4* __restrict__ src,
   uint32_t acc = 0;
   const size_t stride = static_cast<size_t>(gridDim.x) * 256;
   size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  // Four independent 16-byte loads in flight per lane.
-  for (; i + 3 * stride < n_vec; i += 4 * stride) {
-    const U32x4 a = __builtin_nontemporal_load(src + i);
-    const U32x4 b = __builtin_nontemporal_load(src + i + stride);
-    const U32x4 c = __builtin_nontemporal_load(src + i + 2 * stride);
-    const U32x4 d = __builtin_nontemporal_load(src + i + 3 * stride);
-    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
-    acc ^= c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  // Eight independent 16-byte loads in flight per lane; consecutive workgroups read
+  // consecutive 4 KB, so the requests in flight at any moment cover one contiguous region.
+  constexpr int kInFlight = 8;
+  for (; i + (kInFlight - 1) * stride < n_vec; i += kInFlight * stride) {
+    U32x4 v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
   for (; i < n_vec; i += stride) {
     const U32x4 a = src[i];
@@ -126,8 +127,11 @@ hipError_t LaunchReadProbe(const void* src, size_t bytes, uint32_t* sink,
                            hipStream_t stream) {
   const size_t n_vec = bytes / 16;
   if (n_vec == 0) return hipSuccess;
-  size_t blocks = (n_vec + 256 * 4 - 1) / (256 * 4);
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  // At most three workgroups per compute unit: measured, a larger grid loses 20% (the
+  // requests in flight then spread over too many DRAM pages at once).
+  size_t blocks = (n_vec + 256 * 8 - 1) / (256 * 8);
+  const size_t resident = static_cast<size_t>(DeviceComputeUnits()) * 3;
+  if (blocks > resident) blocks = resident;
   hipLaunchKernelGGL(ReadProbe, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
                      stream, static_cast<const U32x4*>(src), n_vec, sink);
   return hipGetLastError();
