@@ -841,6 +841,10 @@ void PlanGemv(int type, const GemvLaunch& launch, GemvParams* prm) {
   const uint32_t nb = launch.blocks_per_row;
   prm->row_bytes = nb * BlockBytes(type);
   prm->cols = nb * 256;
+  // Blocks of a row per wave pass: the largest power of two (up to 16) dividing nb, so
+  // that no lane idles.  (Measured alternative for rows with an odd factor, e.g. 2560 =
+  // 10 blocks as 2 blocks x 5 passes: one padded pass of 16 block slots with 6 idle gives
+  // more, shorter work items but ran 20-60% slower at every column count.)
   uint32_t bpp_log2 = 0;
   while (bpp_log2 < 4 && (nb & ((2u << bpp_log2) - 1)) == 0) ++bpp_log2;
   prm->bpp_log2 = bpp_log2;
