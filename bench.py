@@ -123,6 +123,32 @@ class DecodeSet:
         x = self.act if stage == "ffn_down" else self.x
         capi.gemv_dev([capi.whole(m) for m in mats], x, 1, self.out[stage])
 
+    def fused_stage(self, stage, copy):
+        """The stage with the elementwise step Decoder::Step runs before it taken into
+        the product: residual add + RmsNorm before attention_in, ffn_in and lm_head,
+        SwiGLU before ffn_down (which then reads ffn_in's [gate | up] row)."""
+        capi, cfg = self.capi, self.cfg
+        if not hasattr(self, "norm"):
+            import numpy as np
+            self.norm = capi.DeviceBuffer.from_array(np.ones(cfg.HIDDEN2, dtype=np.float32))
+            self.residual = [capi.DeviceBuffer(4 * cfg.HIDDEN2) for _ in range(3)]
+        if stage == "lm_head":
+            mats = [self.heads[copy % len(self.heads)]]
+        else:
+            layer = self.layers[copy % len(self.layers)]
+            mats = [layer[n] for n in cfg.CONFIG2_STAGES[stage]]
+        parts = [capi.whole(m) for m in mats]
+        if stage == "mixer_out":
+            capi.gemv_dev(parts, self.x, 1, self.out[stage])
+        elif stage == "ffn_down":
+            capi.gemv_fused_dev(parts, capi.swiglu_prologue(), self.out["ffn_in"], 1,
+                                self.out[stage])
+        else:
+            slot = {"attention_in": 0, "ffn_in": 1, "lm_head": 2}[stage]
+            delta = self.out["ffn_down" if slot != 1 else "mixer_out"]
+            prologue = capi.resnorm_prologue(self.norm, 1e-6, delta, self.residual[slot])
+            capi.gemv_fused_dev(parts, prologue, self.x, 1, self.out[stage])
+
     def step(self, copy):
         for stage in self.cfg.CONFIG2_STAGES:
             self.stage(stage, copy)
@@ -195,6 +221,19 @@ def run_details(capi, cfg, synth, decode, args):
         n = 6 if stage == "lm_head" else 30
         ms = time_recorded(capi, [lambda i=i, s=stage: decode.stage(s, i) for i in range(n)])
         report(stage, nbytes, ms)
+
+    log("config 2, the same stages with the decoder's elementwise steps inside the product "
+        "(residual add + RmsNorm before attention_in / ffn_in / lm_head, SwiGLU before "
+        "ffn_down):")
+    fused_total = 0.0
+    for stage, names in cfg.CONFIG2_STAGES.items():
+        nbytes = sum(cfg.CONFIG2[n].nbytes for n in names)
+        n = 6 if stage == "lm_head" else 30
+        ms = time_recorded(capi, [lambda i=i, s=stage: decode.fused_stage(s, i)
+                                  for i in range(n)])
+        fused_total += ms
+        report(stage + (" (plain)" if stage == "mixer_out" else " (fused)"), nbytes, ms)
+    log(f"  sum of the five stages with the steps inside: {fused_total * 1e3:.2f} us")
 
     log("read probe (plain streaming read, the ceiling a kernel can reach):")
     probe = capi.DeviceBuffer(1 << 30)

@@ -87,6 +87,8 @@ SIGNATURES = {
                                 _P, C.c_int, _P]),
     "gufo_hip_gemv_dev": (C.c_int, [C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ), C.c_int,
                                     _P, C.c_int, _P]),
+    "gufo_hip_gemv_fused_dev": (C.c_int, [C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ),
+                                          C.c_int, _P, _P, C.c_int, _P]),
     "gufo_hip_argmax_dev": (C.c_int, [_P, _SZ, C.POINTER(C.c_int64)]),
     "gufo_hip_route_topk": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
     "gufo_hip_route_topk_dev": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
@@ -270,6 +272,40 @@ def gemv_dev(parts: Sequence[Part], x: DeviceBuffer, tokens: int, y: DeviceBuffe
     handles, first, rows, n = _parts_arrays(parts)
     _check(load_library().gufo_hip_gemv_dev(handles, first, rows, n, C.c_void_p(x.ptr),
                                             tokens, C.c_void_p(y.ptr)))
+
+
+PROLOGUE_PLAIN, PROLOGUE_SWIGLU, PROLOGUE_RESNORM = 0, 1, 2
+
+
+class Prologue(C.Structure):
+    """struct gufo_hip_prologue: what a product does to its activation rows first."""
+    _fields_ = [("kind", C.c_int), ("delta_dev", C.c_void_p), ("norm_weight_dev", C.c_void_p),
+                ("eps", C.c_float), ("residual_out_dev", C.c_void_p),
+                ("normed_out_dev", C.c_void_p)]
+
+
+def _dev_ptr(buf: "DeviceBuffer | None"):
+    return None if buf is None else C.c_void_p(buf.ptr)
+
+
+def swiglu_prologue() -> Prologue:
+    return Prologue(PROLOGUE_SWIGLU, None, None, 0.0, None, None)
+
+
+def resnorm_prologue(norm_weight: DeviceBuffer, eps: float, delta: DeviceBuffer | None = None,
+                     residual_out: DeviceBuffer | None = None,
+                     normed_out: DeviceBuffer | None = None) -> Prologue:
+    return Prologue(PROLOGUE_RESNORM, _dev_ptr(delta), _dev_ptr(norm_weight), eps,
+                    _dev_ptr(residual_out), _dev_ptr(normed_out))
+
+
+def gemv_fused_dev(parts: Sequence[Part], prologue: Prologue | None, x: DeviceBuffer,
+                   tokens: int, y: DeviceBuffer) -> None:
+    """gemv_dev with the elementwise step before the product taken into its kernel."""
+    handles, first, rows, n = _parts_arrays(parts)
+    _check(load_library().gufo_hip_gemv_fused_dev(
+        handles, first, rows, n, None if prologue is None else C.byref(prologue),
+        C.c_void_p(x.ptr), tokens, C.c_void_p(y.ptr)))
 
 
 def argmax_dev(logits: DeviceBuffer, n: int) -> int:

@@ -204,9 +204,51 @@ int CheckParts(const gufo_hip_matrix* const* parts, const size_t* first_row,
   return GUFO_HIP_OK;
 }
 
+bool Overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
+  if (a == nullptr || b == nullptr) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a);
+  const uintptr_t b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+// The operands of a prologue, checked for a call of `tokens` rows of `cols` values.
+int CheckPrologue(const gufo::GemvPrologue& in, const float* x, const float* y, int tokens,
+                  size_t cols, size_t stride) {
+  if (in.kind == gufo::kProloguePlain || in.kind == gufo::kPrologueSwiGlu) return GUFO_HIP_OK;
+  if (in.kind != gufo::kPrologueResNorm) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "unknown prologue kind %d", in.kind);
+  }
+  if (in.norm_weight == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "the resnorm prologue needs a norm weight");
+  }
+  if (!(in.eps >= 0.0f)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "eps = %g", in.eps);
+  if (!Aligned16(in.delta) || !Aligned16(in.norm_weight) || !Aligned16(in.residual_out) ||
+      !Aligned16(in.normed_out)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "the rows of a resnorm prologue must be 16-byte aligned");
+  }
+  // Workgroup 0 stores these rows while the others still read x, delta and the weight.
+  const size_t bytes = static_cast<size_t>(tokens) * cols * sizeof(float);
+  const size_t y_bytes = static_cast<size_t>(tokens) * stride * sizeof(float);
+  float* const outs[2] = {in.residual_out, in.normed_out};
+  for (float* out : outs) {
+    if (Overlap(out, bytes, x, bytes) || Overlap(out, bytes, in.delta, bytes) ||
+        Overlap(out, bytes, in.norm_weight, cols * sizeof(float)) ||
+        Overlap(out, bytes, y, y_bytes)) {
+      return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                  "residual_out and normed_out must not overlap x, delta, the norm weight "
+                  "or y");
+    }
+  }
+  if (Overlap(in.residual_out, bytes, in.normed_out, bytes)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "residual_out and normed_out overlap");
+  }
+  return GUFO_HIP_OK;
+}
+
 int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
-                  const size_t* n_rows, int n_parts, const float* x, int tokens,
-                  float* y) {
+                  const size_t* n_rows, int n_parts, const gufo::GemvPrologue& in,
+                  const float* x, int tokens, float* y) {
   size_t stride = 0;
   GUFO_TRY(CheckParts(parts, first_row, n_rows, n_parts, tokens, &stride));
   if (tokens == 0 || stride == 0) return GUFO_HIP_OK;
@@ -217,6 +259,16 @@ int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
   }
   const size_t cols = parts[0]->cols;
+  GUFO_TRY(CheckPrologue(in, x, y, tokens, cols, stride));
+  if (in.kind != gufo::kProloguePlain) {
+    for (int p = 0; p < n_parts; ++p) {
+      if (parts[p]->type == gufo::kTypeF32) {
+        return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                    "part %d holds fp32 rows, which take no prologue", p);
+      }
+    }
+  }
+  const size_t x_row_floats = in.kind == gufo::kPrologueSwiGlu ? 2 * cols : cols;
   // Token columns per pass over the weights: what the narrowest type's LDS need
   // allows for rows this wide.
   int per_pass = kMaxGemvTokens;
@@ -254,9 +306,16 @@ int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
       launch.total_rows = total;
       launch.blocks_per_row = static_cast<uint32_t>(cols / gufo::kSuperBlock);
       launch.y_stride = static_cast<uint32_t>(stride);
-      GUFO_HIP_TRY(gufo::LaunchGemv(type, launch, x + static_cast<size_t>(t0) * cols, nt,
-                                    y + static_cast<size_t>(t0) * stride,
-                                    g_state.stream));
+      // The operands of this pass's first token.
+      gufo::GemvPrologue pass_in = in;
+      const size_t row0 = static_cast<size_t>(t0) * cols;
+      if (in.delta != nullptr) pass_in.delta = in.delta + row0;
+      if (in.residual_out != nullptr) pass_in.residual_out = in.residual_out + row0;
+      if (in.normed_out != nullptr) pass_in.normed_out = in.normed_out + row0;
+      GUFO_HIP_TRY(gufo::LaunchGemvFused(type, launch, pass_in,
+                                         x + static_cast<size_t>(t0) * x_row_floats, nt,
+                                         y + static_cast<size_t>(t0) * stride,
+                                         g_state.stream));
     }
   }
   return GUFO_HIP_OK;
@@ -674,7 +733,34 @@ int gufo_hip_gemv_dev(const gufo_hip_matrix* const* parts, const size_t* first_r
                       float* y_dev) {
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
-  return GemvDevLocked(parts, first_row, n_rows, n_parts, x_dev, tokens, y_dev);
+  return GemvDevLocked(parts, first_row, n_rows, n_parts, gufo::GemvPrologue{}, x_dev, tokens,
+                       y_dev);
+}
+
+int gufo_hip_gemv_fused_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                            const size_t* n_rows, int n_parts,
+                            const gufo_hip_prologue* prologue, const float* x_dev, int tokens,
+                            float* y_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  gufo::GemvPrologue in;
+  if (prologue != nullptr) {
+    switch (prologue->kind) {
+      case GUFO_HIP_PROLOGUE_PLAIN: in.kind = gufo::kProloguePlain; break;
+      case GUFO_HIP_PROLOGUE_SWIGLU: in.kind = gufo::kPrologueSwiGlu; break;
+      case GUFO_HIP_PROLOGUE_RESNORM:
+        in.kind = gufo::kPrologueResNorm;
+        in.delta = prologue->delta_dev;
+        in.norm_weight = prologue->norm_weight_dev;
+        in.eps = prologue->eps;
+        in.residual_out = prologue->residual_out_dev;
+        in.normed_out = prologue->normed_out_dev;
+        break;
+      default:
+        return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "unknown prologue kind %d", prologue->kind);
+    }
+  }
+  return GemvDevLocked(parts, first_row, n_rows, n_parts, in, x_dev, tokens, y_dev);
 }
 
 int gufo_hip_gemv(const gufo_hip_matrix* const* parts, const size_t* first_row,
@@ -692,7 +778,7 @@ int gufo_hip_gemv(const gufo_hip_matrix* const* parts, const size_t* first_row,
   const size_t y_bytes = static_cast<size_t>(tokens) * stride * sizeof(float);
   GUFO_TRY(CopyIn(&g_state.stage_x, x_host, x_bytes));
   GUFO_TRY(Reserve(&g_state.stage_y, y_bytes));
-  GUFO_TRY(GemvDevLocked(parts, first_row, n_rows, n_parts,
+  GUFO_TRY(GemvDevLocked(parts, first_row, n_rows, n_parts, gufo::GemvPrologue{},
                          static_cast<const float*>(g_state.stage_x.ptr), tokens,
                          static_cast<float*>(g_state.stage_y.ptr)));
   return CopyOut(y_host, g_state.stage_y.ptr, y_bytes);

@@ -42,6 +42,29 @@ int GemvMaxTokens(int type, uint32_t blocks_per_row);
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream);
 
+// What a dense product does to its activation rows before multiplying: the elementwise
+// steps the reference's decoder runs between its products
+// (src/models/qwen35/decoder.cpp:491-512), and its NPU GEMV fuses as input stages
+// (src/npu/gemv.hpp:58-63).
+constexpr int kProloguePlain = 0;    // x[t] as given
+constexpr int kPrologueSwiGlu = 1;   // x[t] holds [gate | up] (2*cols): silu(gate) * up
+constexpr int kPrologueResNorm = 2;  // RmsNorm(x[t] + delta[t]) * norm_weight
+struct GemvPrologue {
+  int kind = kProloguePlain;
+  // kPrologueResNorm only; token rows are cols floats apart.
+  const float* delta = nullptr;        // added to x before the norm, or null
+  const float* norm_weight = nullptr;  // cols
+  float eps = 0.0f;
+  float* residual_out = nullptr;  // <- x + delta, or null
+  float* normed_out = nullptr;    // <- the normalized rows, or null
+};
+
+// LaunchGemv with a prologue.  K-quant and Q8_0 rows; fp32 rows take kProloguePlain only.
+// The outputs of kPrologueResNorm must not overlap x, delta or each other: other
+// workgroups are still reading those rows when workgroup 0 stores.
+hipError_t LaunchGemvFused(int type, const GemvLaunch& launch, const GemvPrologue& in,
+                           const float* x, int tokens, float* y, hipStream_t stream);
+
 // The same for rows stored as fp32 (LaunchGemv forwards type 0 here).
 hipError_t LaunchGemvF32(const GemvLaunch& launch, const float* x, int tokens, float* y,
                          hipStream_t stream);

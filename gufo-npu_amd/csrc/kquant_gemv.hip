@@ -91,7 +91,14 @@ __device__ __forceinline__ int Dot4(uint32_t codes, uint32_t limbs, int acc) {
                                 false);
 }
 
-__device__ __forceinline__ float Silu(float v) { return v / (1.0f + expf(-v)); }
+// v / (1 + e^-v) through the hardware's exp2 and reciprocal (about one unit in the last
+// place each): every workgroup takes the activation of its whole input row, so the
+// library exp and the exact division would cost the wide down projections a
+// microsecond.  e^-v overflows to +inf for v < -88.7: 1 / inf = 0, the limit.
+__device__ __forceinline__ float Silu(float v) {
+  const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
+  return v * __builtin_amdgcn_rcpf(1.0f + e);
+}
 
 // ---- the quantized activation row ---------------------------------------------
 //
@@ -197,29 +204,94 @@ __device__ __forceinline__ const float* ColumnX(const Columns<NTOK>& col, uint32
   return p;
 }
 
-// The 8 consecutive activations one staging thread handles, as loaded.  With
-// kSwiGlu the row holds [gate | up] (2*cols values) and the activation is
-// silu(gate) * up, the step between an expert's two products
-// (src/models/qwen35/decoder.cpp:547-549 of the reference).  Fetch only issues the
-// loads, so a kernel can have them in flight early; Values waits for them.
-template <bool kSwiGlu>
+// ---- cross-lane sum ----------------------------------------------------------------
+// Sum over a group of `lanes` (4..64, a power of two) consecutive lanes with DPP adds
+// in a fixed order.  The group's last lane ends with the total.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float DppAdd(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xF,
+                                                false);
+  return v + __int_as_float(moved);
+}
+
+__device__ __forceinline__ float GroupTotal(float v, int lanes) {
+  v = DppAdd<0xB1, 0xF>(v);                    // quad_perm [1,0,3,2]
+  v = DppAdd<0x4E, 0xF>(v);                    // quad_perm [2,3,0,1]
+  if (lanes >= 8) v = DppAdd<0x141, 0xF>(v);   // row_half_mirror
+  if (lanes >= 16) v = DppAdd<0x140, 0xF>(v);  // row_mirror
+  if (lanes >= 32) v = DppAdd<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  if (lanes >= 64) v = DppAdd<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+  return v;
+}
+
+// ---- what happens to an activation row on its way in -----------------------------------
+//   kInPlain    the row as given.
+//   kInSwiGlu   the row holds [gate | up] (2*cols values) and the activation is
+//               silu(gate) * up, the step between the two products of a feed-forward
+//               block (src/models/qwen35/decoder.cpp:509-512,547-549 of the reference).
+//   kInResNorm  the activation is RmsNorm(x + delta) * weight: the residual add and the
+//               norm that precede the first product of each half of a decoder layer
+//               (src/models/qwen35/decoder.cpp:491,500-505; RmsNorm is
+//               src/core/vec.hpp:56-63).  Workgroup 0 also stores x + delta and the
+//               normalized row for the steps that follow.
+constexpr int kInPlain = kProloguePlain;
+constexpr int kInSwiGlu = kPrologueSwiGlu;
+constexpr int kInResNorm = kPrologueResNorm;
+
+// The 8 consecutive activations one staging thread handles, as loaded.  Fetch only
+// issues the loads, so a kernel can have them in flight early; Raw and Values wait for
+// them.
+template <int kIn>
 struct Octet {
   float4 lo[2];
-  float4 up[2];
+  float4 up[2];      // kInSwiGlu: the up half; kInResNorm: delta
+  float4 weight[2];  // kInResNorm: the norm weight
 
-  __device__ __forceinline__ void Fetch(const float* row, uint32_t at, uint32_t cols) {
+  // `row` is the token's activation row, `at` the first of the 8 values; `delta_row` the
+  // token's row of the addend (null: none).
+  __device__ __forceinline__ void Fetch(const float* row, uint32_t at, uint32_t cols,
+                                        const float* delta_row, const float* norm_weight) {
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       lo[q] = reinterpret_cast<const float4*>(row + at)[q];
-      if (kSwiGlu) up[q] = reinterpret_cast<const float4*>(row + cols + at)[q];
+      if (kIn == kInSwiGlu) up[q] = reinterpret_cast<const float4*>(row + cols + at)[q];
+      if (kIn == kInResNorm) {
+        up[q] = delta_row != nullptr ? reinterpret_cast<const float4*>(delta_row + at)[q]
+                                     : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        weight[q] = reinterpret_cast<const float4*>(norm_weight + at)[q];
+      }
     }
   }
 
-  __device__ __forceinline__ void Values(float (&v)[8]) const {
+  // kInResNorm: x + delta, the values the norm is taken over.  (x + 0 == x for every x
+  // but -0, whose square and whose product are the same as those of +0.)
+  __device__ __forceinline__ void Raw(float (&v)[8]) const {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      v[4 * q + 0] = lo[q].x + up[q].x;
+      v[4 * q + 1] = lo[q].y + up[q].y;
+      v[4 * q + 2] = lo[q].z + up[q].z;
+      v[4 * q + 3] = lo[q].w + up[q].w;
+    }
+  }
+
+  // The activations.  `inverse_rms` is used by kInResNorm only.
+  __device__ __forceinline__ void Values(float (&v)[8], float inverse_rms) const {
+    if (kIn == kInResNorm) {
+      Raw(v);
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        v[4 * q + 0] = v[4 * q + 0] * inverse_rms * weight[q].x;
+        v[4 * q + 1] = v[4 * q + 1] * inverse_rms * weight[q].y;
+        v[4 * q + 2] = v[4 * q + 2] * inverse_rms * weight[q].z;
+        v[4 * q + 3] = v[4 * q + 3] * inverse_rms * weight[q].w;
+      }
+      return;
+    }
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       float4 f = lo[q];
-      if (kSwiGlu) {
+      if (kIn == kInSwiGlu) {
         const float4 u = up[q];
         f = make_float4(Silu(f.x) * u.x, Silu(f.y) * u.y, Silu(f.z) * u.z, Silu(f.w) * u.w);
       }
@@ -230,6 +302,17 @@ struct Octet {
     }
   }
 };
+
+// Token rows of the kInResNorm operands are `cols` floats apart.
+template <int kIn>
+__device__ __forceinline__ void FetchOctet(Octet<kIn>* piece, const float* row, uint32_t token,
+                                           uint32_t at, uint32_t cols,
+                                           const GemvPrologue& in) {
+  const float* delta_row =
+      kIn == kInResNorm && in.delta != nullptr ? in.delta + static_cast<size_t>(token) * cols
+                                               : nullptr;
+  piece->Fetch(row, at, cols, delta_row, in.norm_weight);
+}
 
 // Which token column and which 8 values of it staging piece `u` is.
 struct OctetIndex {
@@ -255,27 +338,90 @@ __device__ __forceinline__ OctetIndex IndexOctet(uint32_t u, uint32_t octets_per
 // `first` holds the loads of the thread's first piece (u = threadIdx.x), fetched by the
 // caller before it issued its weight loads: memory returns loads in issue order, so
 // this way the wait for x does not also wait for the weights.
-template <int TYPE, int NTOK, bool kSwiGlu>
+//
+// kInResNorm first takes 1 / rms of every token row.  The sum of squares is formed in an
+// order that depends on the row length alone - a thread adds the pieces o = thread,
+// thread + 256, ... of a row, the 64 lanes of a wave are added by GroupTotal, the four
+// waves in order - so a token's activations, and with them its outputs, are the same
+// bits in whichever column of whichever call it travels.  The four wave sums per token
+// pass through the 64 bytes of LDS behind the staged rows.
+template <int TYPE, int NTOK, int kIn>
 __device__ __forceinline__ void StageActivations(const GemvParams& prm,
                                                  const Columns<NTOK>& col,
-                                                 const Octet<kSwiGlu>& first, U32x4* lds) {
+                                                 const GemvPrologue& in,
+                                                 const Octet<kIn>& first, U32x4* lds) {
   constexpr bool kSix = TYPE == kTypeQ6K;
   constexpr uint32_t kSlots = Slots<TYPE>();
   const uint32_t bpp_log2 = prm.bpp_log2;
   const uint32_t positions = 4u << bpp_log2;  // lanes that cover one pass of a row
   const uint32_t octets = prm.launch.blocks_per_row * 32;  // 8-value pieces per token
+  float inverse_rms[NTOK];
+#pragma unroll
+  for (int t = 0; t < NTOK; ++t) inverse_rms[t] = 1.0f;
+  if (kIn == kInResNorm) {
+    float* wave_sums = reinterpret_cast<float*>(
+        lds + static_cast<size_t>(NTOK) * prm.launch.blocks_per_row * 4 * kSlots);
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+      float squares = 0.0f;
+      for (uint32_t o = threadIdx.x; o < octets; o += kThreads) {
+        float r[8];
+        if (t * octets + o == threadIdx.x) {
+          first.Raw(r);
+        } else {
+          Octet<kIn> piece;
+          FetchOctet(&piece, col.x[t], t, o * 8, prm.cols, in);
+          piece.Raw(r);
+        }
+        float of_piece = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) of_piece = Fma(r[c], r[c], of_piece);
+        squares += of_piece;
+      }
+      squares = GroupTotal(squares, 64);
+      if ((threadIdx.x & 63) == 63) wave_sums[t * kWavesPerGroup + (threadIdx.x >> 6)] = squares;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < NTOK; ++t) {
+      float total = wave_sums[t * kWavesPerGroup];
+#pragma unroll
+      for (int w = 1; w < kWavesPerGroup; ++w) total += wave_sums[t * kWavesPerGroup + w];
+      inverse_rms[t] = 1.0f / sqrtf(total / static_cast<float>(prm.cols) + in.eps);
+    }
+  }
+  const bool keeps_rows = kIn == kInResNorm && blockIdx.x == 0 && blockIdx.y == 0;
   for (uint32_t u = threadIdx.x; u < NTOK * octets; u += kThreads) {
     const OctetIndex ix = IndexOctet(u, octets);
     const uint32_t t = ix.token;
     const uint32_t block = ix.block;
     const uint32_t piece = ix.piece;
+    float inverse = inverse_rms[0];
+#pragma unroll
+    for (int i = 1; i < NTOK; ++i) {
+      if (t == static_cast<uint32_t>(i)) inverse = inverse_rms[i];
+    }
     float v[8];
+    float r[8];  // kInResNorm: the row before the norm
     if (u == threadIdx.x) {
-      first.Values(v);
+      first.Values(v, inverse);
+      if (kIn == kInResNorm) first.Raw(r);
     } else {
-      Octet<kSwiGlu> later;
-      later.Fetch(ColumnX<NTOK>(col, t), block * 256 + piece * 8, prm.cols);
-      later.Values(v);
+      Octet<kIn> later;
+      FetchOctet(&later, ColumnX<NTOK>(col, t), t, block * 256 + piece * 8, prm.cols, in);
+      later.Values(v, inverse);
+      if (kIn == kInResNorm) later.Raw(r);
+    }
+    if (keeps_rows) {
+      const size_t at = static_cast<size_t>(t) * prm.cols + block * 256 + piece * 8;
+      if (in.residual_out != nullptr) {
+        reinterpret_cast<float4*>(in.residual_out + at)[0] = make_float4(r[0], r[1], r[2], r[3]);
+        reinterpret_cast<float4*>(in.residual_out + at)[1] = make_float4(r[4], r[5], r[6], r[7]);
+      }
+      if (in.normed_out != nullptr) {
+        reinterpret_cast<float4*>(in.normed_out + at)[0] = make_float4(v[0], v[1], v[2], v[3]);
+        reinterpret_cast<float4*>(in.normed_out + at)[1] = make_float4(v[4], v[5], v[6], v[7]);
+      }
     }
     float gmax = 0.0f;
 #pragma unroll
@@ -585,36 +731,17 @@ struct LdsX {
   }
 };
 
-// ---- cross-lane sum ----------------------------------------------------------------
-// Sum over a group of `lanes` (4..64, a power of two) consecutive lanes with DPP adds
-// in a fixed order.  The group's last lane ends with the total.
-template <int kCtrl, int kRowMask>
-__device__ __forceinline__ float DppAdd(float v) {
-  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRowMask, 0xF,
-                                                false);
-  return v + __int_as_float(moved);
-}
-
-__device__ __forceinline__ float GroupTotal(float v, int lanes) {
-  v = DppAdd<0xB1, 0xF>(v);                    // quad_perm [1,0,3,2]
-  v = DppAdd<0x4E, 0xF>(v);                    // quad_perm [2,3,0,1]
-  if (lanes >= 8) v = DppAdd<0x141, 0xF>(v);   // row_half_mirror
-  if (lanes >= 16) v = DppAdd<0x140, 0xF>(v);  // row_mirror
-  if (lanes >= 32) v = DppAdd<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
-  if (lanes >= 64) v = DppAdd<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
-  return v;
-}
-
 // ---- the product ---------------------------------------------------------------------
 
 // One workgroup's share.  Row group g (16 >> bpp_log2 consecutive flat rows) is
 // visited by one wave; this wave takes groups g_first, g_first + g_stride, ... below
 // g_end.  part_shift is added to every part's row pointer: the byte offset of an
 // expert inside its 3-D tensor (the parts of one launch share the expert stride).
-template <int TYPE, int NTOK, bool kSwiGlu>
+template <int TYPE, int NTOK, int kIn>
 __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NTOK>& col,
-                                         size_t part_shift, uint32_t g_first,
-                                         uint32_t g_stride, uint32_t g_end, U32x4* lds) {
+                                         const GemvPrologue& in, size_t part_shift,
+                                         uint32_t g_first, uint32_t g_stride, uint32_t g_end,
+                                         U32x4* lds) {
   using Raw = typename RawOf<TYPE>::Type;
   using X = typename XOf<TYPE>::Type;
   constexpr int kBlockBytes = BlockBytes(TYPE);
@@ -675,12 +802,13 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
 
   // The thread's first piece of x, then the first weight loads, then the staging:
   // both latencies overlap, and the wait for x does not wait for the weights.
-  Octet<kSwiGlu> first_piece;
+  Octet<kIn> first_piece;
   {
     const uint32_t octets = prm.launch.blocks_per_row * 32;
     if (threadIdx.x < NTOK * octets) {
       const OctetIndex ix = IndexOctet(threadIdx.x, octets);
-      first_piece.Fetch(ColumnX<NTOK>(col, ix.token), ix.block * 256 + ix.piece * 8, prm.cols);
+      FetchOctet(&first_piece, ColumnX<NTOK>(col, ix.token), ix.token,
+                 ix.block * 256 + ix.piece * 8, prm.cols, in);
     }
   }
 #pragma unroll
@@ -689,7 +817,7 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
     issue(d, 0);
   }
 
-  StageActivations<TYPE, NTOK, kSwiGlu>(prm, col, first_piece, lds);
+  StageActivations<TYPE, NTOK, kIn>(prm, col, in, first_piece, lds);
   __syncthreads();
 
   constexpr bool kResident = NTOK <= kResidentColumns;
@@ -753,20 +881,23 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
 
 // Dense product: token t reads x + t*cols and writes y + t*y_stride; the waves of
 // the whole grid share the row groups round robin.
-template <int TYPE, int NTOK>
+// With kInSwiGlu token t's [gate | up] row is x + t*2*cols.
+template <int TYPE, int NTOK, int kIn>
 __global__ __launch_bounds__(kThreads)
 __attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(NTOK)))) void KquantGemvKernel(
-    const GemvParams prm, const float* __restrict__ x, float* __restrict__ y) {
+    const GemvParams prm, const GemvPrologue in, const float* __restrict__ x,
+    float* __restrict__ y) {
   extern __shared__ __align__(16) U32x4 lds[];
   Columns<NTOK> col;
+  const size_t x_row_floats = kIn == kInSwiGlu ? 2 * static_cast<size_t>(prm.cols) : prm.cols;
 #pragma unroll
   for (int t = 0; t < NTOK; ++t) {
-    col.x[t] = x + static_cast<size_t>(t) * prm.cols;
+    col.x[t] = x + static_cast<size_t>(t) * x_row_floats;
     col.y[t] = y + static_cast<size_t>(t) * prm.launch.y_stride;
   }
   const uint32_t wave = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
-  GemvBody<TYPE, NTOK, false>(prm, col, 0, wave, gridDim.x * kWavesPerGroup,
-                              prm.n_groups, lds);
+  GemvBody<TYPE, NTOK, kIn>(prm, col, in, 0, wave, gridDim.x * kWavesPerGroup, prm.n_groups,
+                            lds);
 }
 
 // Expert product: blockIdx.y names a segment, i.e. one routed expert and up to four
@@ -789,8 +920,8 @@ __device__ __forceinline__ void MoeSegmentBody(const GemvParams& prm,
   const size_t shift = static_cast<size_t>(seg.expert) * moe.expert_bytes;
   const uint32_t first = blockIdx.x * kMoeGroupsPerTile;
   const uint32_t end = min(first + kMoeGroupsPerTile, prm.n_groups);
-  GemvBody<TYPE, NTOK, kSwiGlu>(prm, col, shift, first + (threadIdx.x >> 6),
-                                kWavesPerGroup, end, lds);
+  GemvBody<TYPE, NTOK, kSwiGlu ? kInSwiGlu : kInPlain>(
+      prm, col, GemvPrologue{}, shift, first + (threadIdx.x >> 6), kWavesPerGroup, end, lds);
 }
 
 // kMaxTok bounds the pairs of a segment (the launch's token count, at most four):
@@ -868,24 +999,42 @@ hipError_t AllowLargeLds(Kernel kernel, size_t lds_bytes) {
                              static_cast<int>(kGemvMaxLdsBytes));
 }
 
-template <int TYPE, int NTOK>
-hipError_t LaunchDense(const GemvParams& prm, const float* x, float* y, dim3 grid,
-                       size_t lds_bytes, hipStream_t stream) {
-  const hipError_t status = AllowLargeLds(KquantGemvKernel<TYPE, NTOK>, lds_bytes);
+struct DenseCall {
+  GemvParams prm;
+  GemvPrologue in;
+  const float* x;
+  float* y;
+  dim3 grid;
+  size_t lds_bytes;
+  hipStream_t stream;
+};
+
+template <int TYPE, int NTOK, int kIn>
+hipError_t LaunchDense(const DenseCall& call) {
+  const hipError_t status = AllowLargeLds(KquantGemvKernel<TYPE, NTOK, kIn>, call.lds_bytes);
   if (status != hipSuccess) return status;
-  hipLaunchKernelGGL((KquantGemvKernel<TYPE, NTOK>), grid, dim3(kThreads), lds_bytes, stream,
-                     prm, x, y);
+  hipLaunchKernelGGL((KquantGemvKernel<TYPE, NTOK, kIn>), call.grid, dim3(kThreads),
+                     call.lds_bytes, call.stream, call.prm, call.in, call.x, call.y);
   return hipGetLastError();
 }
 
+template <int TYPE, int NTOK>
+hipError_t LaunchColumns(const DenseCall& call) {
+  switch (call.in.kind) {
+    case kInPlain: return LaunchDense<TYPE, NTOK, kInPlain>(call);
+    case kInSwiGlu: return LaunchDense<TYPE, NTOK, kInSwiGlu>(call);
+    case kInResNorm: return LaunchDense<TYPE, NTOK, kInResNorm>(call);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int TYPE>
-hipError_t LaunchTyped(const GemvParams& prm, const float* x, int tokens, float* y,
-                       dim3 grid, size_t lds_bytes, hipStream_t stream) {
+hipError_t LaunchTyped(const DenseCall& call, int tokens) {
   switch (tokens) {
-    case 1: return LaunchDense<TYPE, 1>(prm, x, y, grid, lds_bytes, stream);
-    case 2: return LaunchDense<TYPE, 2>(prm, x, y, grid, lds_bytes, stream);
-    case 3: return LaunchDense<TYPE, 3>(prm, x, y, grid, lds_bytes, stream);
-    case 4: return LaunchDense<TYPE, 4>(prm, x, y, grid, lds_bytes, stream);
+    case 1: return LaunchColumns<TYPE, 1>(call);
+    case 2: return LaunchColumns<TYPE, 2>(call);
+    case 3: return LaunchColumns<TYPE, 3>(call);
+    case 4: return LaunchColumns<TYPE, 4>(call);
     default: return hipErrorInvalidValue;
   }
 }
@@ -930,26 +1079,43 @@ int GemvMaxTokens(int type, uint32_t blocks_per_row) {
 
 hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int tokens,
                       float* y, hipStream_t stream) {
-  if (type == kTypeF32) return LaunchGemvF32(launch, x, tokens, y, stream);
+  return LaunchGemvFused(type, launch, GemvPrologue{}, x, tokens, y, stream);
+}
+
+hipError_t LaunchGemvFused(int type, const GemvLaunch& launch, const GemvPrologue& in,
+                           const float* x, int tokens, float* y, hipStream_t stream) {
+  if (type == kTypeF32) {
+    // The fp32 kernel reads x as it goes and has no staging step to fuse into.
+    if (in.kind != kInPlain) return hipErrorInvalidValue;
+    return LaunchGemvF32(launch, x, tokens, y, stream);
+  }
   if (!ValidLaunch(type, launch) || tokens < 1 ||
       tokens > GemvMaxTokens(type, launch.blocks_per_row)) {
     return hipErrorInvalidValue;
   }
+  if (in.kind == kInResNorm && in.norm_weight == nullptr) return hipErrorInvalidValue;
+  DenseCall call;
+  call.in = in;
+  call.x = x;
+  call.y = y;
+  call.stream = stream;
+  // kInResNorm keeps the four wave sums of every token behind the staged rows.
+  call.lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens) +
+                   (in.kind == kInResNorm ? kMaxGemvTokens * kWavesPerGroup * sizeof(float) : 0);
+  if (call.lds_bytes > kGemvMaxLdsBytes) return hipErrorInvalidValue;
   if (launch.total_rows == 0) return hipSuccess;
-  GemvParams prm;
-  PlanGemv(type, launch, &prm);
-  const size_t lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens);
-  uint32_t blocks = (prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
+  PlanGemv(type, launch, &call.prm);
+  uint32_t blocks = (call.prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
   // Persistent: no more workgroups than are resident at once.
   const uint32_t resident =
       static_cast<uint32_t>(g_compute_units) * WavesPerSimdFor(tokens);
   if (blocks > resident) blocks = resident;
-  const dim3 grid(blocks);
+  call.grid = dim3(blocks);
   switch (type) {
-    case kTypeQ4K: return LaunchTyped<kTypeQ4K>(prm, x, tokens, y, grid, lds_bytes, stream);
-    case kTypeQ5K: return LaunchTyped<kTypeQ5K>(prm, x, tokens, y, grid, lds_bytes, stream);
-    case kTypeQ6K: return LaunchTyped<kTypeQ6K>(prm, x, tokens, y, grid, lds_bytes, stream);
-    case kTypeQ80: return LaunchTyped<kTypeQ80>(prm, x, tokens, y, grid, lds_bytes, stream);
+    case kTypeQ4K: return LaunchTyped<kTypeQ4K>(call, tokens);
+    case kTypeQ5K: return LaunchTyped<kTypeQ5K>(call, tokens);
+    case kTypeQ6K: return LaunchTyped<kTypeQ6K>(call, tokens);
+    case kTypeQ80: return LaunchTyped<kTypeQ80>(call, tokens);
     default: return hipErrorInvalidValue;
   }
 }

@@ -139,6 +139,47 @@ int gufo_hip_gemv_dev(const gufo_hip_matrix* const* parts, const size_t* first_r
                       const size_t* n_rows, int n_parts, const float* x_dev,
                       int tokens, float* y_dev);
 
+/* What a product does to its activation rows before multiplying: the elementwise
+ * steps Decoder::Step runs on the host between its products
+ * (src/models/qwen35/decoder.cpp:491-512), taken into the product's own kernel the way
+ * the reference's NPU GEMV takes them as input stages (Prologue,
+ * src/npu/gemv.hpp:58-63), so that a decoder layer is four launches with nothing
+ * between them.
+ *   PLAIN    x[t] as given (cols values).
+ *   SWIGLU   x[t] holds [gate | up], 2*cols values, e.g. the y row of the product
+ *            before; the activation is silu(gate[i]) * up[i]
+ *            (decoder.cpp:509-512, Silu at :28-33; here x / (1 + exp(-x)) in fp32).
+ *   RESNORM  the activation is RmsNorm(x[t] + delta[t]) * norm_weight, with
+ *            RmsNorm(v)[i] = v[i] * (1 / sqrt(mean(v^2) + eps)) * w[i] in fp32
+ *            (src/core/vec.hpp:56-63): the residual add that ends one half of a layer
+ *            (decoder.cpp:500-502,526-528) and the norm that opens the next (:491,505).
+ *            delta_dev may be NULL (the first layer has nothing to add).  If not NULL,
+ *            residual_out_dev receives x + delta (the new residual stream) and
+ *            normed_out_dev the normalized rows (for the router and the experts of a
+ *            mixture layer, which read the same input); token rows of all four are
+ *            cols floats apart, 16-byte aligned, and the two outputs must not overlap
+ *            x, delta, the weight, y or each other.
+ * Rows of fp32 matrices take PLAIN only.  Column t of a multi-token call stays
+ * bit-identical to a one-token call on the same row with every prologue. */
+enum gufo_hip_prologue_kind {
+  GUFO_HIP_PROLOGUE_PLAIN = 0,
+  GUFO_HIP_PROLOGUE_SWIGLU = 1,
+  GUFO_HIP_PROLOGUE_RESNORM = 2
+};
+typedef struct gufo_hip_prologue {
+  int kind;
+  const float* delta_dev;       /* RESNORM: tokens x cols, or NULL */
+  const float* norm_weight_dev; /* RESNORM: cols */
+  float eps;                    /* RESNORM: Config::rms_eps */
+  float* residual_out_dev;      /* RESNORM: tokens x cols, or NULL */
+  float* normed_out_dev;        /* RESNORM: tokens x cols, or NULL */
+} gufo_hip_prologue;
+/* gufo_hip_gemv_dev with a prologue (NULL: PLAIN). */
+int gufo_hip_gemv_fused_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                            const size_t* n_rows, int n_parts,
+                            const gufo_hip_prologue* prologue, const float* x_dev,
+                            int tokens, float* y_dev);
+
 /* Greedy pick over logits, std::max_element's rule: the first maximum wins
  * (src/core/sampling.cpp:327-329).  `index` receives the position. */
 int gufo_hip_argmax_dev(const float* logits_dev, size_t n, int64_t* index_host);

@@ -455,6 +455,35 @@ int64_t gufo_oracle_argmax(const float* v, size_t n) {
 
 float gufo_oracle_silu(float x) { return x / (1.0f + expf(-x)); }
 
+void gufo_oracle_rms_norm(const float* x, const float* w, size_t n, float eps,
+                          float* out) {
+  float lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  size_t i = 0;
+  for (; i + 8 <= n; i += 8) {
+    for (int l = 0; l < 8; ++l) lanes[l] += x[i + l] * x[i + l];
+  }
+  float total = 0.0f;
+  for (int l = 0; l < 8; ++l) total += lanes[l];
+  for (; i < n; ++i) total += x[i] * x[i];
+  const float inv = 1.0f / sqrtf(total / (float)n + eps);
+  for (i = 0; i < n; ++i) out[i] = x[i] * inv * w[i];
+}
+
+void gufo_oracle_res_norm(const float* x, const float* delta, const float* w, size_t n,
+                          float eps, float* residual, float* normed) {
+  for (size_t i = 0; i < n; ++i) normed[i] = delta != NULL ? x[i] + delta[i] : x[i];
+  if (residual != NULL) memcpy(residual, normed, n * sizeof(float));
+  gufo_oracle_rms_norm(normed, w, n, eps, normed);
+}
+
+void gufo_oracle_swiglu(const float* gate_up, size_t f, float* act) {
+  for (size_t i = 0; i < f; ++i) {
+    const float g = gate_up[i];
+    const float sigmoid = 1.0f / (1.0f + expf(-g));
+    act[i] = g * sigmoid * gate_up[f + i];
+  }
+}
+
 /* ---- Expert grouping and the routed FFN: reference.cpp:514-607 ----------- */
 
 int gufo_oracle_moe_group(const int* chosen, int tokens, int k, int experts,

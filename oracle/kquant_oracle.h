@@ -24,6 +24,12 @@
  *                      floor case; compiled reference Route
  *   moe_group/moe_ffn  grouped result equals the per-token ungrouped result
  *   argmax             first maximum wins (std::max_element semantics)
+ *   rms_norm/res_norm  closed form in double (x / sqrt(mean x^2 + eps) * w); constant
+ *                      rows, whose norm is sign(c) / sqrt(1 + eps / c^2); invariance to
+ *                      scaling the row by a power of two when eps = 0; compiled
+ *                      reference vec::RmsNorm
+ *   swiglu             closed form in double; silu(0) = 0, silu(x) -> x for large x,
+ *                      silu(-x) = silu(x) - x
  */
 #ifndef GUFO_KQUANT_ORACLE_H_
 #define GUFO_KQUANT_ORACLE_H_
@@ -119,6 +125,23 @@ int gufo_oracle_moe_ffn(const uint8_t* gate, int gate_type, const uint8_t* up,
 
 /* core/simd.hpp:82-84 (Silu) */
 float gufo_oracle_silu(float x);
+
+/* core/vec.hpp:56-63: out[i] = x[i] * inv * w[i], inv = 1 / sqrt(Dot(x,x)/n + eps), all
+ * fp32, Dot in the order of its portable branch (vec.hpp:36-51): eight partial sums by
+ * index mod 8, added in order, then the tail.  out may alias x. */
+void gufo_oracle_rms_norm(const float* x, const float* w, size_t n, float eps,
+                          float* out);
+
+/* The residual add that ends a half layer and the norm that opens the next
+ * (models/qwen35/decoder.cpp:500-505): residual = x + delta (delta NULL: x),
+ * normed = RmsNorm(residual) * w.  residual may be NULL. */
+void gufo_oracle_res_norm(const float* x, const float* delta, const float* w, size_t n,
+                          float eps, float* residual, float* normed);
+
+/* The activation between the two products of the dense feed-forward block
+ * (models/qwen35/decoder.cpp:509-512 with Silu of :28-33, x * (1 / (1 + e^-x))):
+ * act[i] = silu(gate_up[i]) * gate_up[f + i], i < f. */
+void gufo_oracle_swiglu(const float* gate_up, size_t f, float* act);
 
 #ifdef __cplusplus
 }

@@ -69,6 +69,12 @@ def lib() -> C.CDLL:
                                           _P, C.c_int, C.c_int]
         o.gufo_oracle_silu.restype = C.c_float
         o.gufo_oracle_silu.argtypes = [C.c_float]
+        o.gufo_oracle_rms_norm.restype = None
+        o.gufo_oracle_rms_norm.argtypes = [_P, _P, _SZ, C.c_float, _P]
+        o.gufo_oracle_res_norm.restype = None
+        o.gufo_oracle_res_norm.argtypes = [_P, _P, _P, _SZ, C.c_float, _P, _P]
+        o.gufo_oracle_swiglu.restype = None
+        o.gufo_oracle_swiglu.argtypes = [_P, _SZ, _P]
         _oracle = o
     return _oracle
 
@@ -94,6 +100,8 @@ def ref() -> C.CDLL:
         r.ref_route.argtypes = [_P, C.c_int, C.c_int, _P, _P]
         r.ref_silu.restype = C.c_float
         r.ref_silu.argtypes = [C.c_float]
+        r.ref_rms_norm.restype = None
+        r.ref_rms_norm.argtypes = [_P, _P, C.c_int, C.c_float, _P]
         r.ref_shared_expert_scale.restype = C.c_float
         r.ref_shared_expert_scale.argtypes = [C.c_float]
         r.ref_default_threads.restype = C.c_int
@@ -223,6 +231,42 @@ def moe_ffn(gate, gate_type, up, up_type, down, down_type, experts, hidden, ffn,
 
 def silu(x: float) -> float:
     return lib().gufo_oracle_silu(x)
+
+
+def rms_norm(x: np.ndarray, w: np.ndarray, eps: float, use_ref: bool = False) -> np.ndarray:
+    """RmsNorm of one row (core/vec.hpp:56-63)."""
+    x = _f32(x)
+    w = _f32(w)
+    out = np.empty_like(x)
+    if use_ref:
+        ref().ref_rms_norm(_p(x), _p(w), x.size, eps, _p(out))
+    else:
+        lib().gufo_oracle_rms_norm(_p(x), _p(w), x.size, eps, _p(out))
+    return out
+
+
+def res_norm(x: np.ndarray, delta, w: np.ndarray, eps: float):
+    """(residual, normed) of tokens x n rows: residual = x + delta, normed = RmsNorm(residual)
+    (models/qwen35/decoder.cpp:500-505).  delta may be None."""
+    x = np.atleast_2d(_f32(x))
+    w = _f32(w)
+    d = None if delta is None else np.atleast_2d(_f32(delta))
+    residual = np.empty_like(x)
+    normed = np.empty_like(x)
+    for t in range(x.shape[0]):
+        lib().gufo_oracle_res_norm(_p(x[t]), None if d is None else _p(d[t]), _p(w),
+                                   x.shape[1], eps, _p(residual[t]), _p(normed[t]))
+    return residual, normed
+
+
+def swiglu(gate_up: np.ndarray) -> np.ndarray:
+    """silu(gate) * up of tokens x 2f rows [gate | up] (models/qwen35/decoder.cpp:509-512)."""
+    g = np.atleast_2d(_f32(gate_up))
+    f = g.shape[1] // 2
+    act = np.empty((g.shape[0], f), dtype=np.float32)
+    for t in range(g.shape[0]):
+        lib().gufo_oracle_swiglu(_p(g[t]), f, _p(act[t]))
+    return act
 
 
 def rel_l2(got: np.ndarray, want: np.ndarray) -> float:

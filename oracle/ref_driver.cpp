@@ -30,6 +30,7 @@
 #include "core/quant.hpp"
 #include "core/simd.hpp"
 #include "core/thread_pool.hpp"
+#include "core/vec.hpp"
 #include "models/qwen35/gguf_dot.hpp"
 #include "models/qwen35/moe.hpp"
 
@@ -95,6 +96,11 @@ void ref_route(const float* logits, int experts, int k, int* chosen,
 
 // core/simd.hpp:82-84: x / (1 + e^-x) in fp32.
 float ref_silu(float x) { return gufo_npu::simd::Silu(x); }
+
+// core/vec.hpp:56-63, in the AVX2 order of vec::Dot this build selects.
+void ref_rms_norm(const float* x, const float* w, int n, float eps, float* out) {
+  gufo_npu::vec::RmsNorm(x, w, n, eps, out);
+}
 
 float ref_shared_expert_scale(float logit) {
   return gufo_npu::qwen35::SharedExpertScale(logit);
