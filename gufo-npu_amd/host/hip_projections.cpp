@@ -191,6 +191,37 @@ void HipProjections::Apply(Stage stage, int layer, const float* x, int tokens, f
                       x, tokens, y));
 }
 
+void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
+                                 float* y) const {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  if (parts == nullptr || parts->empty()) {
+    throw std::logic_error("qwen35: no weights for this stage and layer");
+  }
+  std::vector<const gufo_hip_matrix*> handles;
+  std::vector<std::size_t> first;
+  std::vector<std::size_t> rows;
+  for (const Matrix& m : *parts) {
+    handles.push_back(m.handle);
+    first.push_back(0);
+    rows.push_back(m.rows);
+  }
+  gufo_hip_prologue prologue = {};
+  switch (in.prologue) {
+    case Prologue::kPlain: prologue.kind = GUFO_HIP_PROLOGUE_PLAIN; break;
+    case Prologue::kSwiGlu: prologue.kind = GUFO_HIP_PROLOGUE_SWIGLU; break;
+    case Prologue::kResNorm:
+      prologue.kind = GUFO_HIP_PROLOGUE_RESNORM;
+      prologue.delta_dev = in.delta;
+      prologue.norm_weight_dev = in.norm_weight;
+      prologue.eps = in.eps;
+      prologue.residual_out_dev = in.residual;
+      prologue.normed_out_dev = in.normed;
+      break;
+  }
+  Check(gufo_hip_gemv_fused_dev(handles.data(), first.data(), rows.data(),
+                                static_cast<int>(handles.size()), &prologue, in.x, tokens, y));
+}
+
 void HipProjections::ApplyExpert(Stage stage, int layer, int expert, const float* x, int tokens,
                                  float* y) const {
   const Layer& l = layers_.at(static_cast<std::size_t>(layer));

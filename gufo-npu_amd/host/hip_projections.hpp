@@ -108,6 +108,29 @@ public:
   std::size_t StageInputs(Stage stage, int layer) const;
   std::size_t StageOutputs(Stage stage, int layer) const;
 
+  // A stage on rows that stay in device memory, with the elementwise step the decoder
+  // runs before it taken into the product - the reference's NPU products work the same
+  // way (npu::Prologue and Q4nxGemv::Run(x, y, residual, tokens),
+  // src/npu/gemv.hpp:58-63,146-150).  All pointers are device memory
+  // (gufo_hip_malloc); the call is enqueued, not waited for.
+  enum class Prologue {
+    kPlain,    // x: tokens x StageInputs
+    kSwiGlu,   // x: tokens x 2*StageInputs rows [gate | up] -> silu(gate) * up
+               // (decoder.cpp:509-512); the kFfnIn output feeds kFfnDown directly
+    kResNorm,  // RmsNorm(x + delta) * norm_weight (decoder.cpp:491,500-505); x + delta
+               // goes to `residual`, the normalized rows to `normed` (either may be null)
+  };
+  struct DeviceInput {
+    Prologue prologue = Prologue::kPlain;
+    const float* x = nullptr;
+    const float* delta = nullptr;        // kResNorm, may be null
+    const float* norm_weight = nullptr;  // kResNorm
+    float eps = 0.0f;                    // kResNorm: Config::rms_eps
+    float* residual = nullptr;
+    float* normed = nullptr;
+  };
+  void ApplyDevice(Stage stage, int layer, const DeviceInput& in, int tokens, float* y) const;
+
   // qwen35::Route (src/models/qwen35/moe.cpp:16-42) on the device.
   void Route(const float* logits, int tokens, int k, int* chosen, float* weights) const;
   // The routed experts of one MoE layer in one call: what Decoder::MoeFfn /

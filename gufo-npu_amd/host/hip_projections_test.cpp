@@ -15,11 +15,13 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <new>
 #include <random>
 #include <stdexcept>
 #include <string>
 #include <vector>
 
+#include "gufo_hip.h"
 #include "hip_projections.hpp"
 #include "kquant_oracle.h"
 
@@ -338,6 +340,108 @@ void RunMoe(std::mt19937& rng) {
          Throws<std::runtime_error>([&] { HipProjections p(bad); }));
 }
 
+// Rows of floats in device memory.
+class DeviceRows {
+public:
+  explicit DeviceRows(std::size_t n) : n_(n) {
+    void* p = nullptr;
+    if (gufo_hip_malloc(&p, n * sizeof(float)) != GUFO_HIP_OK) throw std::bad_alloc();
+    data_ = static_cast<float*>(p);
+  }
+  explicit DeviceRows(const std::vector<float>& host) : DeviceRows(host.size()) {
+    gufo_hip_memcpy_h2d(data_, host.data(), n_ * sizeof(float));
+  }
+  ~DeviceRows() { gufo_hip_free(data_); }
+  DeviceRows(const DeviceRows&) = delete;
+  DeviceRows& operator=(const DeviceRows&) = delete;
+  float* get() const { return data_; }
+  std::vector<float> Download() const {
+    std::vector<float> host(n_);
+    gufo_hip_memcpy_d2h(host.data(), data_, n_ * sizeof(float));
+    return host;
+  }
+
+private:
+  std::size_t n_;
+  float* data_ = nullptr;
+};
+
+// The second half of a dense decoder layer on rows that stay on the device
+// (src/models/qwen35/decoder.cpp:500-512,526-528 of the reference): the residual add
+// and RmsNorm inside the kFfnIn product, SwiGLU inside the kFfnDown product - two
+// launches - against the same steps taken one at a time by the checker.
+void RunDeviceChain(std::mt19937& rng) {
+  const std::size_t hidden = 512, ffn = 768;
+  const float eps = 1e-6f;
+  const Weights gate = RandomWeights(GUFO_ORACLE_Q4_K, ffn, hidden, rng);
+  const Weights up = RandomWeights(GUFO_ORACLE_Q4_K, ffn, hidden, rng);
+  const Weights down = RandomWeights(GUFO_ORACLE_Q6_K, hidden, ffn, rng);
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  LayerTensors layer;
+  layer.ffn_in = {AsTensor("blk.0.ffn_gate.weight", gate), AsTensor("blk.0.ffn_up.weight", up)};
+  layer.ffn_down = {AsTensor("blk.0.ffn_down.weight", down)};
+  model.layers.push_back(layer);
+  const HipProjections proj(model);
+
+  for (const int tokens : {1, 2, 4}) {
+    const auto n = static_cast<std::size_t>(tokens);
+    const auto h = RandomActivations(n * hidden, rng);
+    const auto mixer_out = RandomActivations(n * hidden, rng, 0.5f);
+    auto norm_weight = RandomActivations(hidden, rng, 0.1f);
+    for (auto& w : norm_weight) w += 1.0f;
+
+    std::vector<float> want_h(n * hidden), normed(n * hidden), act(n * ffn);
+    for (std::size_t t = 0; t < n; ++t) {
+      gufo_oracle_res_norm(&h[t * hidden], &mixer_out[t * hidden], norm_weight.data(), hidden,
+                           eps, &want_h[t * hidden], &normed[t * hidden]);
+    }
+    auto gate_up = ExpectedWhole({&gate, &up}, normed, tokens);
+    // Synthetic weights are not zero-mean: keep the activation of order one.
+    for (auto& v : gate_up) v *= 1.0f / 64;
+    for (std::size_t t = 0; t < n; ++t) {
+      gufo_oracle_swiglu(&gate_up[t * 2 * ffn], ffn, &act[t * ffn]);
+    }
+    const auto want_y = ExpectedWhole({&down}, act, tokens);
+
+    const DeviceRows d_h(h), d_mixer(mixer_out), d_weight(norm_weight);
+    const DeviceRows d_residual(n * hidden), d_gate_up(n * 2 * ffn), d_y(n * hidden);
+    HipProjections::DeviceInput in;
+    in.prologue = HipProjections::Prologue::kResNorm;
+    in.x = d_h.get();
+    in.delta = d_mixer.get();
+    in.norm_weight = d_weight.get();
+    in.eps = eps;
+    in.residual = d_residual.get();
+    proj.ApplyDevice(Stage::kFfnIn, 0, in, tokens, d_gate_up.get());
+    auto scaled = d_gate_up.Download();
+    for (auto& v : scaled) v *= 1.0f / 64;
+    const DeviceRows d_scaled(scaled);
+    HipProjections::DeviceInput act_in;
+    act_in.prologue = HipProjections::Prologue::kSwiGlu;
+    act_in.x = d_scaled.get();
+    proj.ApplyDevice(Stage::kFfnDown, 0, act_in, tokens, d_y.get());
+
+    const std::string tag = " tokens=" + std::to_string(tokens);
+    Report("ApplyDevice kResNorm residual row is x + delta exactly" + tag,
+           d_residual.Download() == want_h);
+    double err = RelL2(scaled, gate_up);
+    Report("ApplyDevice kFfnIn with kResNorm" + tag, err <= kTolerance, err);
+    err = RelL2(d_y.Download(), want_y);
+    Report("ApplyDevice kFfnDown with kSwiGlu" + tag, err <= 2 * kTolerance, err);
+  }
+  const DeviceRows d_x(std::vector<float>(hidden, 1.0f)), d_y(2 * ffn);
+  HipProjections::DeviceInput no_weight;
+  no_weight.prologue = HipProjections::Prologue::kResNorm;
+  no_weight.x = d_x.get();
+  Report("kResNorm without a norm weight throws std::invalid_argument",
+         Throws<std::invalid_argument>(
+             [&] { proj.ApplyDevice(Stage::kFfnIn, 0, no_weight, 1, d_y.get()); }));
+  Report("ApplyDevice on a missing stage throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.ApplyDevice(Stage::kRouter, 0, no_weight, 1, d_y.get());
+         }));
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -346,6 +450,7 @@ int main(int argc, char** argv) {
   try {
     RunDense(rng);
     RunMoe(rng);
+    RunDeviceChain(rng);
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAIL: unexpected exception: %s\n", e.what());
     return 1;
