@@ -54,8 +54,22 @@ def build_host_tests() -> list[Path]:
     return [target]
 
 
+def build_model_library() -> Path:
+    """The host side above the C-ABI as a library of its own: the GGUF reader, the stage
+    table, the Projections adapter and their extern "C" layer (include/gufo_hip_model.h).
+    Host code only (g++); links libgufo_hip.so."""
+    target = LIB_DIR / "libgufo_hip_model.so"
+    _run(["g++", "-std=c++20", "-O2", "-mf16c", "-fPIC", "-shared", "-Wall", "-Wextra",
+          "-I", str(ROOT / "include"), "-I", str(HOST), "-o", str(target),
+          str(HOST / "model_capi.cpp"), str(HOST / "gguf_model.cpp"),
+          str(HOST / "hip_projections.cpp"), "-L", str(LIB_DIR), "-lgufo_hip",
+          "-Wl,-rpath,$ORIGIN", "-pthread"])
+    return target
+
+
 def build_all() -> None:
     build_library()
+    build_model_library()
     build_host_tests()
 
 

@@ -100,6 +100,15 @@ def ref() -> C.CDLL:
         r.ref_route.argtypes = [_P, C.c_int, C.c_int, _P, _P]
         r.ref_silu.restype = C.c_float
         r.ref_silu.argtypes = [C.c_float]
+        r.ref_last_error.restype = C.c_char_p
+        r.ref_gguf_open.restype = _P
+        r.ref_gguf_open.argtypes = [C.c_char_p]
+        r.ref_gguf_close.restype = None
+        r.ref_gguf_close.argtypes = [_P]
+        r.ref_gguf_config.restype = None
+        r.ref_gguf_config.argtypes = [_P, _P, _P]
+        r.ref_gguf_apply.restype = C.c_int
+        r.ref_gguf_apply.argtypes = [_P, C.c_int, C.c_int, C.c_int, _P, C.c_int, _P, C.c_int]
         r.ref_rms_norm.restype = None
         r.ref_rms_norm.argtypes = [_P, _P, C.c_int, C.c_float, _P]
         r.ref_shared_expert_scale.restype = C.c_float
@@ -267,6 +276,147 @@ def swiglu(gate_up: np.ndarray) -> np.ndarray:
     for t in range(g.shape[0]):
         lib().gufo_oracle_swiglu(_p(g[t]), f, _p(act[t]))
     return act
+
+
+CONFIG_FIELDS = ("layers", "mtp_layers", "hidden", "ffn", "vocab", "full_attention_interval",
+                 "heads", "kv_heads", "head_dim", "rope_dim", "conv_kernel", "linear_key_heads",
+                 "linear_value_heads", "linear_head_dim", "experts", "experts_used",
+                 "expert_ffn", "shared_expert_ffn", "tied_embeddings", "has_mtp_layer")
+
+
+class RefModel:
+    """A GGUF file opened by the compiled reference: its reader, ReadConfig and
+    GgufProjections (core/gguf.cpp, models/qwen35/config.cpp, gguf_projections.cpp)."""
+
+    def __init__(self, path):
+        self.handle = ref().ref_gguf_open(str(path).encode())
+        if not self.handle:
+            raise RuntimeError(ref().ref_last_error().decode())
+        fields = np.zeros(len(CONFIG_FIELDS), dtype=np.int32)
+        eps = np.zeros(1, dtype=np.float32)
+        ref().ref_gguf_config(self.handle, _p(fields), _p(eps))
+        self.config = dict(zip(CONFIG_FIELDS, (int(v) for v in fields)))
+        self.config["rms_eps"] = float(eps[0])
+
+    def apply(self, stage: int, layer: int, x: np.ndarray, outputs: int, expert: int = -1,
+              exact: bool = False) -> np.ndarray:
+        """Projections::Apply (ApplyExpert with expert >= 0) on tokens x inputs rows."""
+        x = np.atleast_2d(_f32(x))
+        y = np.empty((x.shape[0], outputs), dtype=np.float32)
+        if ref().ref_gguf_apply(self.handle, stage, layer, expert, _p(x), x.shape[0], _p(y),
+                                int(exact)) != 0:
+            raise RuntimeError(ref().ref_last_error().decode())
+        return y
+
+    def close(self):
+        if self.handle:
+            ref().ref_gguf_close(self.handle)
+            self.handle = None
+
+
+# ---- which tensors make up which stage -------------------------------------------------
+# Stage numbers of qwen35::Stage (models/qwen35/projections.hpp:14-39).
+(STAGE_LINEAR_IN, STAGE_ATTENTION_IN, STAGE_MIXER_OUT, STAGE_FFN_IN, STAGE_FFN_DOWN,
+ STAGE_LM_HEAD, STAGE_ROUTER, STAGE_EXPERT_IN, STAGE_EXPERT_DOWN, STAGE_MTP_IN) = range(10)
+
+
+def stage_parts(config: dict, stage: int, layer: int, expert: int = -1):
+    """The row ranges of one stage as (tensor name, first row, rows or None for all), in
+    output order: the table the GgufProjections constructor builds and Apply /
+    ApplyExpert read (models/qwen35/gguf_projections.cpp:100-237).  `config` holds the
+    Config fields (CONFIG_FIELDS).  An empty list: the layer has no such stage."""
+    c = config
+    moe = c["experts"] > 0
+    full = layer >= c["layers"] or (layer + 1) % c["full_attention_interval"] == 0
+    p = f"blk.{layer}."
+    tail = "_shexp.weight" if moe else ".weight"
+    if stage == STAGE_LM_HEAD:
+        return [("token_embd.weight" if c["tied_embeddings"] else "output.weight", 0, None)]
+    if stage == STAGE_LINEAR_IN:
+        names = [] if full else ["attn_qkv", "attn_gate", "ssm_alpha", "ssm_beta"]
+        return [(p + n + ".weight", 0, None) for n in names]
+    if stage == STAGE_ATTENTION_IN:
+        names = ["attn_q", "attn_k", "attn_v"] if full else []
+        return [(p + n + ".weight", 0, None) for n in names]
+    if stage == STAGE_MIXER_OUT:
+        return [(p + ("attn_output" if full else "ssm_out") + ".weight", 0, None)]
+    if stage == STAGE_FFN_IN:
+        return [(p + "ffn_gate" + tail, 0, None), (p + "ffn_up" + tail, 0, None)]
+    if stage == STAGE_FFN_DOWN:
+        return [(p + "ffn_down" + tail, 0, None)]
+    if stage == STAGE_ROUTER:
+        if not moe:
+            return []
+        return [(p + "ffn_gate_inp.weight", 0, None), (p + "ffn_gate_inp_shexp.weight", 0, None)]
+    if stage == STAGE_MTP_IN:
+        return [(p + "nextn.eh_proj.weight", 0, None)] if layer >= c["layers"] else []
+    if stage == STAGE_EXPERT_IN and moe and 0 <= expert < c["experts"]:
+        f = c["expert_ffn"]
+        return [(p + "ffn_gate_exps.weight", expert * f, f),
+                (p + "ffn_up_exps.weight", expert * f, f)]
+    if stage == STAGE_EXPERT_DOWN and moe and 0 <= expert < c["experts"]:
+        h = c["hidden"]
+        return [(p + "ffn_down_exps.weight", expert * h, h)]
+    return []
+
+
+def _full_attention(c: dict, layer: int) -> bool:
+    return layer >= c["layers"] or (layer + 1) % c["full_attention_interval"] == 0
+
+
+def stage_inputs(c: dict, stage: int, layer: int) -> int:
+    """StageInputs (models/qwen35/reference.cpp:609-624): values per token row read."""
+    if stage == STAGE_MIXER_OUT:
+        return (c["heads"] * c["head_dim"] if _full_attention(c, layer)
+                else c["linear_value_heads"] * c["linear_head_dim"])
+    if stage == STAGE_FFN_DOWN:
+        return c["shared_expert_ffn"] if c["experts"] > 0 else c["ffn"]
+    if stage == STAGE_EXPERT_DOWN:
+        return c["expert_ffn"]
+    if stage == STAGE_MTP_IN:
+        return 2 * c["hidden"]
+    return c["hidden"]
+
+
+def stage_outputs(c: dict, stage: int, layer: int) -> int:
+    """StageOutputs (models/qwen35/reference.cpp:626-648): values per token row written."""
+    key_dim = c["linear_key_heads"] * c["linear_head_dim"]
+    value_dim = c["linear_value_heads"] * c["linear_head_dim"]
+    ffn = c["shared_expert_ffn"] if c["experts"] > 0 else c["ffn"]
+    return {
+        STAGE_LINEAR_IN: 2 * key_dim + 2 * value_dim + 2 * c["linear_value_heads"],
+        STAGE_ATTENTION_IN: 2 * c["heads"] * c["head_dim"] + 2 * c["kv_heads"] * c["head_dim"],
+        STAGE_MIXER_OUT: c["hidden"], STAGE_FFN_DOWN: c["hidden"],
+        STAGE_EXPERT_DOWN: c["hidden"], STAGE_MTP_IN: c["hidden"],
+        STAGE_FFN_IN: 2 * ffn, STAGE_LM_HEAD: c["vocab"], STAGE_ROUTER: c["experts"] + 1,
+        STAGE_EXPERT_IN: 2 * c["expert_ffn"],
+    }[stage]
+
+
+def widen_16bit(ggml_type: int, data: np.ndarray) -> tuple[int, np.ndarray]:
+    """F16 / BF16 rows as F32 rows (quant::Dequantize, core/quant.cpp:240-262): what the
+    reference does with such tensors before it multiplies them."""
+    raw = np.ascontiguousarray(data).view(np.uint8).reshape(data.shape[0], -1)
+    if ggml_type == 1:
+        wide = raw.view(np.float16).astype(np.float32)
+    elif ggml_type == 30:
+        wide = (raw.view(np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+    else:
+        return ggml_type, raw
+    return F32, np.ascontiguousarray(wide).view(np.uint8).reshape(data.shape[0], -1)
+
+
+def stage_apply(config: dict, tensors: dict, stage: int, layer: int, x: np.ndarray,
+                expert: int = -1, precision: str = "double", threads: int = 4) -> np.ndarray:
+    """Projections::Apply / ApplyExpert by the checker.  tensors: name -> (ggml type,
+    bytes[rows_total, row_bytes])."""
+    parts = []
+    for name, first, rows in stage_parts(config, stage, layer, expert):
+        ggml_type, data = widen_16bit(*tensors[name])
+        parts.append((ggml_type, data, first, data.shape[0] if rows is None else rows))
+    if not parts:
+        raise LookupError("qwen35: no weights for this stage and layer")
+    return matmul(parts, np.atleast_2d(_f32(x)), precision=precision, threads=threads)
 
 
 def rel_l2(got: np.ndarray, want: np.ndarray) -> float:

@@ -19,18 +19,26 @@
 //     y[t*stride + offset + r], the loop of GgufProjections::MatMul
 //     (models/qwen35/gguf_projections.cpp:239-286); the loop itself is restated
 //     here because MatMul is a private member that needs a whole model file.
+//   * ref_gguf_* open a GGUF file with the reference's reader (core/gguf.cpp), read its
+//     Config (models/qwen35/config.cpp) and run the reference's GgufProjections itself
+//     (models/qwen35/gguf_projections.cpp: stage table, shape checks, MatMul) - with a
+//     model file, synthetic or real, nothing of that class needs restating.
 #include <algorithm>
 #include <cstddef>
 #include <cstdint>
 #include <memory>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "core/cpus.hpp"
 #include "core/quant.hpp"
 #include "core/simd.hpp"
+#include "core/gguf.hpp"
 #include "core/thread_pool.hpp"
 #include "core/vec.hpp"
+#include "models/qwen35/config.hpp"
+#include "models/qwen35/gguf_projections.hpp"
 #include "models/qwen35/gguf_dot.hpp"
 #include "models/qwen35/moe.hpp"
 
@@ -159,6 +167,83 @@ int ref_matmul(int n_parts, const std::uint8_t* const* data, const int* types,
     }
   });
   return 0;
+}
+
+// ---- a whole model file through the reference's own classes ---------------------------
+
+namespace {
+
+struct RefModel {
+  std::unique_ptr<gufo_npu::gguf::File> file;
+  gufo_npu::qwen35::Config config;
+  std::unique_ptr<gufo_npu::qwen35::GgufProjections> fused;  // Precision::kFloat
+  std::unique_ptr<gufo_npu::qwen35::GgufProjections> exact;  // Precision::kDouble
+};
+
+thread_local std::string g_ref_error;
+
+}  // namespace
+
+const char* ref_last_error() { return g_ref_error.c_str(); }
+
+// nullptr (and ref_last_error) when the reference rejects the file.
+void* ref_gguf_open(const char* path) {
+  try {
+    auto model = std::make_unique<RefModel>();
+    model->file = gufo_npu::gguf::File::Open(path);
+    model->config = gufo_npu::qwen35::ReadConfig(*model->file);
+    using gufo_npu::qwen35::GgufProjections;
+    model->fused = std::make_unique<GgufProjections>(*model->file,
+                                                     GgufProjections::Precision::kFloat);
+    model->exact = std::make_unique<GgufProjections>(*model->file,
+                                                     GgufProjections::Precision::kDouble);
+    return model.release();
+  } catch (const std::exception& e) {
+    g_ref_error = e.what();
+    return nullptr;
+  }
+}
+
+void ref_gguf_close(void* handle) { delete static_cast<RefModel*>(handle); }
+
+// The Config fields, in the order of models/qwen35/config.hpp:13-52:
+// layers, mtp_layers, hidden, ffn, vocab, full_attention_interval, heads, kv_heads,
+// head_dim, rope_dim, conv_kernel, linear_key_heads, linear_value_heads,
+// linear_head_dim, experts, experts_used, expert_ffn, shared_expert_ffn,
+// tied_embeddings, has_mtp_layer (HasMtpLayer).
+void ref_gguf_config(void* handle, int* out, float* rms_eps) {
+  const RefModel& m = *static_cast<RefModel*>(handle);
+  const auto& c = m.config;
+  const int fields[20] = {c.layers, c.mtp_layers, c.hidden, c.ffn, c.vocab,
+                          c.full_attention_interval, c.heads, c.kv_heads, c.head_dim,
+                          c.rope_dim, c.conv_kernel, c.linear_key_heads,
+                          c.linear_value_heads, c.linear_head_dim, c.experts,
+                          c.experts_used, c.expert_ffn, c.shared_expert_ffn,
+                          c.tied_embeddings ? 1 : 0,
+                          gufo_npu::qwen35::HasMtpLayer(*m.file, c) ? 1 : 0};
+  std::copy(fields, fields + 20, out);
+  *rms_eps = c.rms_eps;
+}
+
+// Stage numbers follow qwen35::Stage (models/qwen35/projections.hpp:14-39).  expert < 0:
+// Apply; otherwise ApplyExpert.  Returns 0, or -1 with ref_last_error set when the
+// reference throws.
+int ref_gguf_apply(void* handle, int stage, int layer, int expert, const float* x, int tokens,
+                   float* y, int exact) {
+  const RefModel& m = *static_cast<RefModel*>(handle);
+  const auto& proj = exact != 0 ? *m.exact : *m.fused;
+  const auto s = static_cast<gufo_npu::qwen35::Stage>(stage);
+  try {
+    if (expert < 0) {
+      proj.Apply(s, layer, x, tokens, y);
+    } else {
+      proj.ApplyExpert(s, layer, expert, x, tokens, y);
+    }
+    return 0;
+  } catch (const std::exception& e) {
+    g_ref_error = e.what();
+    return -1;
+  }
 }
 
 }  // extern "C"
