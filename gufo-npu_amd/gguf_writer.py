@@ -56,25 +56,38 @@ class TensorSpec:
     data: np.ndarray      # the bytes as stored, any shape, uint8
 
 
-def write_image(metadata: dict, tensors: list[TensorSpec]) -> bytes:
-    """The bytes of a GGUF v3 file holding `metadata` and `tensors`."""
+def _header(metadata: dict, tensors: list[TensorSpec]) -> bytes:
+    """Everything before the data section, padding included."""
     head = bytearray(b"GGUF" + struct.pack("<IQQ", 3, len(tensors), len(metadata)))
     for key, v in metadata.items():
         head += _string(key) + _value(v)
-    offsets, at = [], 0
+    at = 0
     for t in tensors:
-        offsets.append(at)
-        at += (t.data.size + ALIGNMENT - 1) // ALIGNMENT * ALIGNMENT
-    for t, offset in zip(tensors, offsets):
         head += _string(t.name) + struct.pack("<I", len(t.shape))
         head += b"".join(struct.pack("<Q", d) for d in t.shape)
-        head += struct.pack("<IQ", t.ggml_type, offset)
+        head += struct.pack("<IQ", t.ggml_type, at)
+        at += (t.data.size + ALIGNMENT - 1) // ALIGNMENT * ALIGNMENT
     head += b"\0" * (-len(head) % ALIGNMENT)
-    body = bytearray(at)
-    for t, offset in zip(tensors, offsets):
+    return bytes(head)
+
+
+def write_file(path, metadata: dict, tensors: list[TensorSpec]) -> None:
+    """A GGUF v3 file holding `metadata` and `tensors`, streamed tensor by tensor."""
+    with open(path, "wb") as f:
+        f.write(_header(metadata, tensors))
+        for t in tensors:
+            raw = np.ascontiguousarray(t.data).view(np.uint8).reshape(-1)
+            f.write(raw.data)
+            f.write(b"\0" * (-raw.size % ALIGNMENT))
+
+
+def write_image(metadata: dict, tensors: list[TensorSpec]) -> bytes:
+    """The same file as bytes in memory (for small models and for damaging on purpose)."""
+    parts = [_header(metadata, tensors)]
+    for t in tensors:
         raw = np.ascontiguousarray(t.data).view(np.uint8).reshape(-1)
-        body[offset:offset + raw.size] = raw.tobytes()
-    return bytes(head) + bytes(body)
+        parts += [raw.tobytes(), b"\0" * (-raw.size % ALIGNMENT)]
+    return b"".join(parts)
 
 
 # ---- synthetic models ---------------------------------------------------------------
@@ -192,6 +205,32 @@ def model_tensors(spec: ModelSpec) -> list[TensorSpec]:
         add(p + "ffn_gate" + tail, h, spec.ffn_width)
         add(p + "ffn_up" + tail, h, spec.ffn_width)
         add(p + "ffn_down" + tail, spec.ffn_width, h)
+    # The small fp32 tensors of the mixers (src/models/qwen35/decoder.cpp:72-87 of the
+    # reference), so that the reference's own decoder can run on the file.  They are
+    # seeded apart from the projections and do not enter any product of this backend.
+    for il in range(spec.layers + spec.mtp_layers):
+        p = f"blk.{il}."
+        gen = synth.rng(spec.seed + 50_000 + il)
+
+        def small(name, shape, values):
+            out.append(TensorSpec(p + name, F32, shape,
+                                  np.ascontiguousarray(values, dtype=np.float32).view(np.uint8)))
+
+        if spec.is_full_attention(il):
+            for name in ("attn_q_norm.weight", "attn_k_norm.weight"):
+                small(name, (spec.head_dim,),
+                      1.0 + 0.1 * gen.standard_normal(spec.head_dim, dtype=np.float32))
+        else:
+            channels = 2 * spec.key_dim + spec.value_dim
+            small("ssm_conv1d.weight", (4, channels),
+                  0.3 * gen.standard_normal((channels, 4), dtype=np.float32))
+            # A decay rate: negative, so the recurrent state shrinks (decoder.cpp:227).
+            small("ssm_a", (spec.linear_value_heads,),
+                  -np.exp(0.5 * gen.standard_normal(spec.linear_value_heads, dtype=np.float32)))
+            small("ssm_dt.bias", (spec.linear_value_heads,),
+                  0.5 * gen.standard_normal(spec.linear_value_heads, dtype=np.float32))
+            small("ssm_norm.weight", (spec.linear_head_dim,),
+                  1.0 + 0.1 * gen.standard_normal(spec.linear_head_dim, dtype=np.float32))
     return out
 
 
@@ -234,6 +273,10 @@ def model_image(spec: ModelSpec) -> bytes:
     return write_image(model_metadata(spec), model_tensors(spec))
 
 
+def write_model(path, spec: ModelSpec) -> None:
+    write_file(path, model_metadata(spec), model_tensors(spec))
+
+
 # The row types of a real Unsloth "UD-Q4_K_XL" file, in miniature: K-quants for the large
 # projections, Q8_0 here and there, fp32 for the router and the per-head gates, and a
 # 16-bit tensor (which the reference converts to fp32 before multiplying,
@@ -255,6 +298,15 @@ def tiny_dense(seed: int = synth.BASE_SEED + 9000) -> ModelSpec:
     """Four layers (three linear-attention, one full-attention), tied embeddings, one
     MTP layer: the shape of Qwen3.5-2B at 1/4 width."""
     return ModelSpec(architecture="qwen35", layers=4, mtp_layers=1, seed=seed,
+                     types=dict(_MIXED_TYPES))
+
+
+def dense_2b_like(seed: int = synth.BASE_SEED + 9700) -> ModelSpec:
+    """The widths of the 2B decode set at full size: hidden 2048, FFN 6144, 24 layers of
+    which every fourth is full attention, a 151,936-row tied Q6_K head.  About 1.2 GB."""
+    return ModelSpec(architecture="qwen35", layers=24, hidden=2048, ffn=6144, vocab=151936,
+                     heads=8, kv_heads=4, head_dim=128, linear_key_heads=16,
+                     linear_value_heads=16, linear_head_dim=128, seed=seed,
                      types=dict(_MIXED_TYPES))
 
 

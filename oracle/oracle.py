@@ -109,6 +109,16 @@ def ref() -> C.CDLL:
         r.ref_gguf_config.argtypes = [_P, _P, _P]
         r.ref_gguf_apply.restype = C.c_int
         r.ref_gguf_apply.argtypes = [_P, C.c_int, C.c_int, C.c_int, _P, C.c_int, _P, C.c_int]
+        r.ref_decoder_open.restype = _P
+        r.ref_decoder_open.argtypes = [_P, C.c_int, _P, _P, _P]
+        r.ref_decoder_close.restype = None
+        r.ref_decoder_close.argtypes = [_P]
+        r.ref_decoder_step.restype = C.c_int
+        r.ref_decoder_step.argtypes = [_P, C.c_int, _P]
+        r.ref_decoder_reset.restype = None
+        r.ref_decoder_reset.argtypes = [_P]
+        r.ref_decoder_foreign_calls.restype = C.c_long
+        r.ref_decoder_foreign_calls.argtypes = [_P]
         r.ref_rms_norm.restype = None
         r.ref_rms_norm.argtypes = [_P, _P, C.c_int, C.c_float, _P]
         r.ref_shared_expert_scale.restype = C.c_float
@@ -311,6 +321,43 @@ class RefModel:
     def close(self):
         if self.handle:
             ref().ref_gguf_close(self.handle)
+            self.handle = None
+
+
+class RefDecoder:
+    """The reference's Decoder (models/qwen35/decoder.cpp) on a RefModel, over the
+    reference's own GgufProjections ("float" / "double") or over foreign entry points with
+    the signatures of gufo_model_apply / gufo_model_apply_expert: `foreign` is then
+    (model handle, apply function, apply_expert function) as ctypes objects."""
+
+    def __init__(self, model: RefModel, projections: str = "float", foreign=None):
+        self.model = model
+        which = {"float": 0, "double": 1, "foreign": 2}[projections]
+        handle, apply, apply_expert = foreign if foreign is not None else (None, None, None)
+        self.handle = ref().ref_decoder_open(
+            model.handle, which, handle,
+            None if apply is None else C.cast(apply, C.c_void_p),
+            None if apply_expert is None else C.cast(apply_expert, C.c_void_p))
+        if not self.handle:
+            raise RuntimeError(ref().ref_last_error().decode())
+
+    def step(self, token: int) -> np.ndarray:
+        """Decoder::Step: the logits after `token` at the decoder's position."""
+        logits = np.empty(self.model.config["vocab"], dtype=np.float32)
+        if ref().ref_decoder_step(self.handle, int(token), _p(logits)) != 0:
+            raise RuntimeError(ref().ref_last_error().decode())
+        return logits
+
+    def reset(self) -> None:
+        ref().ref_decoder_reset(self.handle)
+
+    @property
+    def foreign_calls(self) -> int:
+        return int(ref().ref_decoder_foreign_calls(self.handle))
+
+    def close(self) -> None:
+        if self.handle:
+            ref().ref_decoder_close(self.handle)
             self.handle = None
 
 

@@ -23,6 +23,12 @@
 //     Config (models/qwen35/config.cpp) and run the reference's GgufProjections itself
 //     (models/qwen35/gguf_projections.cpp: stage table, shape checks, MatMul) - with a
 //     model file, synthetic or real, nothing of that class needs restating.
+//   * ref_decoder_* run the reference's Decoder (models/qwen35/decoder.cpp: embedding,
+//     norms, mixers, residuals, the MoE loop) over a Projections of the caller's choice:
+//     the reference's GgufProjections in either precision, or ForeignProjections, a
+//     Projections whose two methods forward to a pair of C function pointers.  Handed
+//     gufo_model_apply / gufo_model_apply_expert, that is the reference's own decoder
+//     running on the MI355X backend: the binding a maintainer of the reference adds.
 #include <algorithm>
 #include <cstddef>
 #include <cstdint>
@@ -38,6 +44,7 @@
 #include "core/thread_pool.hpp"
 #include "core/vec.hpp"
 #include "models/qwen35/config.hpp"
+#include "models/qwen35/decoder.hpp"
 #include "models/qwen35/gguf_projections.hpp"
 #include "models/qwen35/gguf_dot.hpp"
 #include "models/qwen35/moe.hpp"
@@ -244,6 +251,99 @@ int ref_gguf_apply(void* handle, int stage, int layer, int expert, const float* 
     g_ref_error = e.what();
     return -1;
   }
+}
+
+// ---- the reference's decoder over any Projections --------------------------------------
+
+namespace {
+
+// qwen35::Projections over C entry points with the signatures of gufo_model_apply and
+// gufo_model_apply_expert (include/gufo_hip_model.h); a non-zero status becomes the
+// exception a consumer of Projections expects.
+class ForeignProjections : public gufo_npu::qwen35::Projections {
+public:
+  using ApplyFn = int (*)(const void*, int, int, const float*, int, float*);
+  using ApplyExpertFn = int (*)(const void*, int, int, int, const float*, int, float*);
+  ForeignProjections(const void* model, ApplyFn apply, ApplyExpertFn apply_expert)
+      : model_(model), apply_(apply), apply_expert_(apply_expert) {}
+  void Apply(gufo_npu::qwen35::Stage stage, int layer, const float* x, int tokens,
+             float* y) const override {
+    ++calls;
+    if (apply_(model_, static_cast<int>(stage), layer, x, tokens, y) != 0) {
+      throw std::runtime_error("foreign Projections::Apply failed");
+    }
+  }
+  void ApplyExpert(gufo_npu::qwen35::Stage stage, int layer, int expert, const float* x,
+                   int tokens, float* y) const override {
+    ++calls;
+    if (apply_expert_(model_, static_cast<int>(stage), layer, expert, x, tokens, y) != 0) {
+      throw std::runtime_error("foreign Projections::ApplyExpert failed");
+    }
+  }
+  mutable long calls = 0;
+
+private:
+  const void* model_;
+  ApplyFn apply_;
+  ApplyExpertFn apply_expert_;
+};
+
+struct RefDecoder {
+  std::unique_ptr<ForeignProjections> foreign;
+  std::unique_ptr<gufo_npu::qwen35::Decoder> decoder;
+  gufo_npu::qwen35::Decoder::State state;
+};
+
+}  // namespace
+
+// which: 0 = GgufProjections fp32, 1 = GgufProjections double, 2 = the foreign entry
+// points.  `model` is a ref_gguf_open handle and must outlive the decoder.
+void* ref_decoder_open(void* model, int which, const void* foreign_model, void* apply,
+                       void* apply_expert) {
+  try {
+    RefModel& m = *static_cast<RefModel*>(model);
+    auto d = std::make_unique<RefDecoder>();
+    const gufo_npu::qwen35::Projections* projections = nullptr;
+    if (which == 2) {
+      d->foreign = std::make_unique<ForeignProjections>(
+          foreign_model, reinterpret_cast<ForeignProjections::ApplyFn>(apply),
+          reinterpret_cast<ForeignProjections::ApplyExpertFn>(apply_expert));
+      projections = d->foreign.get();
+    } else {
+      projections = which == 1 ? m.exact.get() : m.fused.get();
+    }
+    d->decoder = std::make_unique<gufo_npu::qwen35::Decoder>(*m.file, *projections);
+    d->state = d->decoder->NewState();
+    return d.release();
+  } catch (const std::exception& e) {
+    g_ref_error = e.what();
+    return nullptr;
+  }
+}
+
+void ref_decoder_close(void* handle) { delete static_cast<RefDecoder*>(handle); }
+
+// Decoder::Step at the decoder's own position; copies the vocab logits out.
+int ref_decoder_step(void* handle, int token, float* logits) {
+  RefDecoder& d = *static_cast<RefDecoder*>(handle);
+  try {
+    const std::vector<float>& out = d.decoder->Step(token, d.state);
+    std::copy(out.begin(), out.end(), logits);
+    return 0;
+  } catch (const std::exception& e) {
+    g_ref_error = e.what();
+    return -1;
+  }
+}
+
+void ref_decoder_reset(void* handle) {
+  RefDecoder& d = *static_cast<RefDecoder*>(handle);
+  d.state = d.decoder->NewState();
+}
+
+long ref_decoder_foreign_calls(void* handle) {
+  const RefDecoder& d = *static_cast<RefDecoder*>(handle);
+  return d.foreign ? d.foreign->calls : 0;
 }
 
 }  // extern "C"

@@ -37,12 +37,15 @@ def test_shape_and_resident_bytes(opened, oracle):
     for field, value in zip(oracle.CONFIG_FIELDS, golden["config_fields"]):
         assert model.shape[field] == int(value), field
     # Every projection tensor is resident; 16-bit tensors count at their fp32 size.
-    want = 0
+    config = dict(zip(oracle.CONFIG_FIELDS, (int(v) for v in golden["config_fields"])))
     tensors = gguf_cases.tensors_by_name(spec)
-    for name, (ggml_type, data) in tensors.items():
-        if name.endswith("norm.weight") or (name == "token_embd.weight"
-                                            and not spec.tied_embeddings):
-            continue
+    names = {oracle.stage_parts(config, oracle.STAGE_LM_HEAD, -1)[0][0]}
+    for layer in range(spec.layers + spec.mtp_layers):
+        for stage in range(10):
+            names.update(part[0] for part in oracle.stage_parts(config, stage, layer, expert=0))
+    want = 0
+    for name in names:
+        ggml_type, data = tensors[name]
         want += data.size * (2 if ggml_type in (1, 30) else 1)
     assert model.weight_bytes == want
 
