@@ -235,6 +235,27 @@ def run_details(capi, cfg, synth, decode, args):
         report(stage + (" (plain)" if stage == "mixer_out" else " (fused)"), nbytes, ms)
     log(f"  sum of the five stages with the steps inside: {fused_total * 1e3:.2f} us")
 
+    log("config 2, greedy decoding: the head product and the pick of its first maximum:")
+    index = capi.DeviceBuffer(8)
+    head_bytes = cfg.CONFIG2["lm_head"].nbytes
+    ms_head = time_recorded(capi, [lambda i=i: decode.stage("lm_head", i) for i in range(6)])
+    capi.synchronize()
+    # The separate pick copies its result to the host, which a recording cannot hold:
+    # timed from the host, launch and copy latency included.
+    reps = 50
+    start = time.perf_counter()
+    for _ in range(reps):
+        capi.argmax_dev(decode.out["lm_head"], cfg.CONFIG2["lm_head"].rows)
+    ms_pick_sync = (time.perf_counter() - start) * 1e3 / reps
+    ms_fused = time_recorded(capi, [lambda i=i: capi.gemv_argmax_dev(
+        [capi.whole(decode.heads[i % len(decode.heads)])], None, decode.x, 1, index)
+        for i in range(6)])
+    report("lm_head, logits stored", head_bytes, ms_head)
+    log(f"    + separate pick over the stored logits (2 launches, result copied to the host, "
+        f"synchronous): {ms_pick_sync * 1e3:.1f} us")
+    report("lm_head with the pick inside", head_bytes, ms_fused)
+    index.free()
+
     log("read probe (plain streaming read, the ceiling a kernel can reach):")
     probe = capi.DeviceBuffer(1 << 30)
     sink = capi.DeviceBuffer(64)

@@ -89,6 +89,9 @@ SIGNATURES = {
                                     _P, C.c_int, _P]),
     "gufo_hip_gemv_fused_dev": (C.c_int, [C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ),
                                           C.c_int, _P, _P, C.c_int, _P]),
+    "gufo_hip_gemv_argmax_dev": (C.c_int, [C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ),
+                                           C.c_int, _P, _P, C.c_int, _P]),
+    "gufo_hip_matrix_gather_rows": (C.c_int, [_P, _P, _SZ, C.POINTER(_P)]),
     "gufo_hip_argmax_dev": (C.c_int, [_P, _SZ, C.POINTER(C.c_int64)]),
     "gufo_hip_route_topk": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
     "gufo_hip_route_topk_dev": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
@@ -229,6 +232,18 @@ class Matrix:
                                                    C.byref(r), C.byref(c), C.byref(b)))
         return t.value, r.value, c.value, b.value
 
+    def gather_rows(self, rows) -> "Matrix":
+        """A new resident matrix of the given rows of this one, in that order."""
+        ids = np.ascontiguousarray(rows, dtype=np.int64)
+        handle = C.c_void_p()
+        _check(load_library().gufo_hip_matrix_gather_rows(C.c_void_p(self.handle), _ptr(ids),
+                                                          ids.size, C.byref(handle)))
+        picked = Matrix.__new__(Matrix)
+        picked.type, picked.rows, picked.cols = self.type, int(ids.size), self.cols
+        picked.handle = handle.value
+        picked.nbytes = self.nbytes // max(self.rows, 1) * int(ids.size)
+        return picked
+
     def destroy(self) -> None:
         if self.handle:
             _check(load_library().gufo_hip_matrix_destroy(C.c_void_p(self.handle)))
@@ -306,6 +321,16 @@ def gemv_fused_dev(parts: Sequence[Part], prologue: Prologue | None, x: DeviceBu
     _check(load_library().gufo_hip_gemv_fused_dev(
         handles, first, rows, n, None if prologue is None else C.byref(prologue),
         C.c_void_p(x.ptr), tokens, C.c_void_p(y.ptr)))
+
+
+def gemv_argmax_dev(parts: Sequence[Part], prologue: Prologue | None, x: DeviceBuffer,
+                    tokens: int, index: DeviceBuffer) -> None:
+    """The product with the greedy pick inside: index[t] (int64, device) = position of the
+    first maximum of y[t]; y is not stored."""
+    handles, first, rows, n = _parts_arrays(parts)
+    _check(load_library().gufo_hip_gemv_argmax_dev(
+        handles, first, rows, n, None if prologue is None else C.byref(prologue),
+        C.c_void_p(x.ptr), tokens, C.c_void_p(index.ptr)))
 
 
 def argmax_dev(logits: DeviceBuffer, n: int) -> int:

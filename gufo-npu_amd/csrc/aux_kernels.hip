@@ -6,29 +6,6 @@
 namespace gufo {
 namespace {
 
-struct Best {
-  float value;
-  uint32_t index;
-};
-
-// The better of two candidates under std::max_element's rule (first maximum
-// wins): the larger value, the lower index on equal values
-// (src/core/sampling.cpp:327-329 of the reference).
-__device__ __forceinline__ Best Better(Best a, Best b) {
-  const bool take_b = b.value > a.value || (b.value == a.value && b.index < a.index);
-  return take_b ? b : a;
-}
-
-__device__ __forceinline__ Best WaveBest(Best v) {
-  for (int off = 32; off > 0; off >>= 1) {
-    Best o;
-    o.value = __shfl_xor(v.value, off, 64);
-    o.index = __shfl_xor(v.index, off, 64);
-    v = Better(v, o);
-  }
-  return v;
-}
-
 __device__ __forceinline__ Best BlockBest(Best v) {
   __shared__ Best per_wave[4];
   v = WaveBest(v);

@@ -132,7 +132,11 @@ void Release(Scratch* s) {
 constexpr size_t kArgmaxPartialBytes = static_cast<size_t>(gufo::kArgmaxBlocks) * 8;
 constexpr size_t kArgmaxResultOffset = kArgmaxPartialBytes;
 constexpr size_t kMoeHeaderOffset = kArgmaxResultOffset + 64;
-constexpr size_t kSmallBytes = kMoeHeaderOffset + 64;
+// The product with the pick inside: per-workgroup candidates of up to four tokens (at
+// most kPickGroups workgroups per launch).
+constexpr size_t kPickGroups = 1024;
+constexpr size_t kPickPartialOffset = kMoeHeaderOffset + 64;
+constexpr size_t kSmallBytes = kPickPartialOffset + kMaxGemvTokens * kPickGroups * 8;
 
 // Device addresses of the grouping tables inside State::moe_tables.
 struct MoeTablePointers {
@@ -318,6 +322,82 @@ int GemvDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
                                          g_state.stream));
     }
   }
+  return GUFO_HIP_OK;
+}
+
+int ToPrologue(const gufo_hip_prologue* prologue, gufo::GemvPrologue* in) {
+  *in = gufo::GemvPrologue{};
+  if (prologue == nullptr) return GUFO_HIP_OK;
+  switch (prologue->kind) {
+    case GUFO_HIP_PROLOGUE_PLAIN: in->kind = gufo::kProloguePlain; break;
+    case GUFO_HIP_PROLOGUE_SWIGLU: in->kind = gufo::kPrologueSwiGlu; break;
+    case GUFO_HIP_PROLOGUE_RESNORM:
+      in->kind = gufo::kPrologueResNorm;
+      in->delta = prologue->delta_dev;
+      in->norm_weight = prologue->norm_weight_dev;
+      in->eps = prologue->eps;
+      in->residual_out = prologue->residual_out_dev;
+      in->normed_out = prologue->normed_out_dev;
+      break;
+    default:
+      return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "unknown prologue kind %d", prologue->kind);
+  }
+  return GUFO_HIP_OK;
+}
+
+// The product and the greedy pick over each of its rows: index[t] = position of the first
+// maximum of y[t].  The pick rides inside the product's kernel when the call is a single
+// launch of the quantized kernels; otherwise the product goes into library scratch and
+// the pick kernels read it.
+int PickDevLocked(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                  const size_t* n_rows, int n_parts, const gufo::GemvPrologue& in,
+                  const float* x, int tokens, int64_t* index) {
+  size_t stride = 0;
+  GUFO_TRY(CheckParts(parts, first_row, n_rows, n_parts, tokens, &stride));
+  if (tokens == 0) return GUFO_HIP_OK;
+  if (stride == 0) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "no output rows to pick from");
+  if (x == nullptr || index == nullptr) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x or index is null");
+  }
+  if (in.kind == gufo::kPrologueSwiGlu) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "the pick takes the plain and resnorm prologues");
+  }
+  const size_t cols = parts[0]->cols;
+  const int type = parts[0]->type;
+  bool one_launch = type != gufo::kTypeF32 && n_parts <= kMaxGemvParts &&
+                    tokens <= gufo::GemvMaxTokens(type, static_cast<uint32_t>(cols / 256)) &&
+                    gufo::GemvPickPartialBytes(tokens) <= kMaxGemvTokens * kPickGroups * 8;
+  for (int p = 1; p < n_parts; ++p) one_launch = one_launch && parts[p]->type == type;
+  if (!one_launch) {
+    GUFO_TRY(Reserve(&g_state.stage_y, static_cast<size_t>(tokens) * stride * sizeof(float)));
+    float* y = static_cast<float*>(g_state.stage_y.ptr);
+    GUFO_TRY(GemvDevLocked(parts, first_row, n_rows, n_parts, in, x, tokens, y));
+    for (int t = 0; t < tokens; ++t) {
+      GUFO_HIP_TRY(gufo::LaunchArgmax(y + static_cast<size_t>(t) * stride, stride,
+                                      g_state.small.ptr, index + t, g_state.stream));
+    }
+    return GUFO_HIP_OK;
+  }
+  if (!Aligned16(x)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "x must be 16-byte aligned");
+  GUFO_TRY(CheckPrologue(in, x, nullptr, tokens, cols, stride));
+  GemvLaunch launch;
+  std::memset(&launch, 0, sizeof launch);
+  size_t offset = 0;
+  for (int p = 0; p < n_parts; ++p) {
+    launch.part[p].rows = parts[p]->data + first_row[p] * parts[p]->row_bytes;
+    launch.part[p].n_rows = static_cast<uint32_t>(n_rows[p]);
+    launch.part[p].y_offset = static_cast<uint32_t>(offset);
+    offset += n_rows[p];
+  }
+  launch.n_parts = static_cast<uint32_t>(n_parts);
+  launch.total_rows = static_cast<uint32_t>(stride);
+  launch.blocks_per_row = static_cast<uint32_t>(cols / gufo::kSuperBlock);
+  launch.y_stride = static_cast<uint32_t>(stride);
+  uint8_t* small = static_cast<uint8_t*>(g_state.small.ptr);
+  gufo::GemvPick pick;
+  pick.partial = small + kPickPartialOffset;
+  pick.index = index;
+  GUFO_HIP_TRY(gufo::LaunchGemvPick(type, launch, in, x, tokens, pick, g_state.stream));
   return GUFO_HIP_OK;
 }
 
@@ -744,23 +824,66 @@ int gufo_hip_gemv_fused_dev(const gufo_hip_matrix* const* parts, const size_t* f
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
   gufo::GemvPrologue in;
-  if (prologue != nullptr) {
-    switch (prologue->kind) {
-      case GUFO_HIP_PROLOGUE_PLAIN: in.kind = gufo::kProloguePlain; break;
-      case GUFO_HIP_PROLOGUE_SWIGLU: in.kind = gufo::kPrologueSwiGlu; break;
-      case GUFO_HIP_PROLOGUE_RESNORM:
-        in.kind = gufo::kPrologueResNorm;
-        in.delta = prologue->delta_dev;
-        in.norm_weight = prologue->norm_weight_dev;
-        in.eps = prologue->eps;
-        in.residual_out = prologue->residual_out_dev;
-        in.normed_out = prologue->normed_out_dev;
-        break;
-      default:
-        return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "unknown prologue kind %d", prologue->kind);
+  GUFO_TRY(ToPrologue(prologue, &in));
+  return GemvDevLocked(parts, first_row, n_rows, n_parts, in, x_dev, tokens, y_dev);
+}
+
+int gufo_hip_gemv_argmax_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                             const size_t* n_rows, int n_parts,
+                             const gufo_hip_prologue* prologue, const float* x_dev, int tokens,
+                             int64_t* index_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  gufo::GemvPrologue in;
+  GUFO_TRY(ToPrologue(prologue, &in));
+  return PickDevLocked(parts, first_row, n_rows, n_parts, in, x_dev, tokens, index_dev);
+}
+
+int gufo_hip_matrix_gather_rows(const gufo_hip_matrix* src, const int64_t* rows_host,
+                                size_t n, gufo_hip_matrix** out) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (out == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null out pointer");
+  *out = nullptr;
+  if (src == nullptr || (rows_host == nullptr && n != 0)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "null matrix or row list");
+  }
+  for (size_t i = 0; i < n; ++i) {
+    if (rows_host[i] < 0 || static_cast<uint64_t>(rows_host[i]) >= src->rows) {
+      return Fail(GUFO_HIP_ERR_OUT_OF_RANGE, "row %lld of a matrix with %zu rows",
+                  static_cast<long long>(rows_host[i]), src->rows);
     }
   }
-  return GemvDevLocked(parts, first_row, n_rows, n_parts, in, x_dev, tokens, y_dev);
+  gufo_hip_matrix* m = new (std::nothrow) gufo_hip_matrix(*src);
+  if (m == nullptr) return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "host allocation failed");
+  m->rows = n;
+  m->bytes = n * src->row_bytes;
+  m->data = nullptr;
+  hipError_t status = hipMalloc(reinterpret_cast<void**>(&m->data), m->bytes + 64);
+  if (status != hipSuccess) {
+    delete m;
+    return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "hipMalloc of %zu bytes: %s", n * src->row_bytes,
+                hipGetErrorString(status));
+  }
+  // One device copy per run of consecutive rows (a draft vocabulary is mostly runs).
+  for (size_t i = 0; i < n && status == hipSuccess;) {
+    size_t run = 1;
+    while (i + run < n && rows_host[i + run] == rows_host[i] + static_cast<int64_t>(run)) ++run;
+    status = hipMemcpyAsync(m->data + i * src->row_bytes,
+                            src->data + static_cast<size_t>(rows_host[i]) * src->row_bytes,
+                            run * src->row_bytes, hipMemcpyDeviceToDevice, g_state.stream);
+    i += run;
+  }
+  if (status == hipSuccess) status = hipMemsetAsync(m->data + m->bytes, 0, 64, g_state.stream);
+  if (status == hipSuccess) status = hipStreamSynchronize(g_state.stream);
+  if (status != hipSuccess) {
+    (void)hipFree(m->data);
+    delete m;
+    return Fail(GUFO_HIP_ERR_RUNTIME, "gathering rows: %s", hipGetErrorString(status));
+  }
+  ++g_state.live_matrices;
+  *out = m;
+  return GUFO_HIP_OK;
 }
 
 int gufo_hip_gemv(const gufo_hip_matrix* const* parts, const size_t* first_row,

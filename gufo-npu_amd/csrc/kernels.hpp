@@ -44,7 +44,7 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
 
 // What a dense product does to its activation rows before multiplying: the elementwise
 // steps the reference's decoder runs between its products
-// (src/models/qwen35/decoder.cpp:491-512), and its NPU GEMV fuses as input stages
+// (src/models/qwen35/decoder.cpp:493-521), and its NPU GEMV fuses as input stages
 // (src/npu/gemv.hpp:58-63).
 constexpr int kProloguePlain = 0;    // x[t] as given
 constexpr int kPrologueSwiGlu = 1;   // x[t] holds [gate | up] (2*cols): silu(gate) * up
@@ -64,6 +64,22 @@ struct GemvPrologue {
 // workgroups are still reading those rows when workgroup 0 stores.
 hipError_t LaunchGemvFused(int type, const GemvLaunch& launch, const GemvPrologue& in,
                            const float* x, int tokens, float* y, hipStream_t stream);
+
+// The greedy pick taken inside the product: instead of storing y, every workgroup keeps
+// the best (value, position) of the outputs it forms per token, and a one-workgroup-per-
+// token kernel behind it takes the best of those - the head's logits never reach memory
+// (the draft head of the reference's NPU decoder feeds std::max_element the same way,
+// src/models/qwen36_35b_a3b/npu_decoder.cpp:968-973).
+struct GemvPick {
+  void* partial = nullptr;   // GemvPickPartialBytes(tokens) bytes
+  int64_t* index = nullptr;  // tokens results: position of the first maximum of y[t]
+  float* value = nullptr;    // tokens maxima, or null
+};
+size_t GemvPickPartialBytes(int tokens);
+// One product launch only: K-quant or Q8_0 rows, tokens within GemvMaxTokens.
+hipError_t LaunchGemvPick(int type, const GemvLaunch& launch, const GemvPrologue& in,
+                          const float* x, int tokens, const GemvPick& pick,
+                          hipStream_t stream);
 
 // The same for rows stored as fp32 (LaunchGemv forwards type 0 here).
 hipError_t LaunchGemvF32(const GemvLaunch& launch, const float* x, int tokens, float* y,

@@ -103,4 +103,31 @@ __device__ __forceinline__ float GroupSum(float v, int width) {
   return v;
 }
 
+// A candidate of the greedy pick: a value and where it stands.
+struct Best {
+  float value;
+  uint32_t index;
+};
+constexpr uint32_t kNoIndex = 0xFFFFFFFFu;
+
+// The better of two candidates under std::max_element's rule (first maximum
+// wins): the larger value, the lower index on equal values
+// (src/core/sampling.cpp:327-329 of the reference).  A total order on (value, index)
+// pairs without NaN, so the result does not depend on the order of reduction; a NaN
+// never replaces anything.
+__device__ __forceinline__ Best Better(Best a, Best b) {
+  const bool take_b = b.value > a.value || (b.value == a.value && b.index < a.index);
+  return take_b ? b : a;
+}
+
+__device__ __forceinline__ Best WaveBest(Best v) {
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o;
+    o.value = __shfl_xor(v.value, off, 64);
+    o.index = __shfl_xor(v.index, off, 64);
+    v = Better(v, o);
+  }
+  return v;
+}
+
 }  // namespace gufo

@@ -228,10 +228,10 @@ __device__ __forceinline__ float GroupTotal(float v, int lanes) {
 //   kInPlain    the row as given.
 //   kInSwiGlu   the row holds [gate | up] (2*cols values) and the activation is
 //               silu(gate) * up, the step between the two products of a feed-forward
-//               block (src/models/qwen35/decoder.cpp:509-512,547-549 of the reference).
+//               block (src/models/qwen35/decoder.cpp:511-514,547-549 of the reference).
 //   kInResNorm  the activation is RmsNorm(x + delta) * weight: the residual add and the
 //               norm that precede the first product of each half of a decoder layer
-//               (src/models/qwen35/decoder.cpp:491,500-505; RmsNorm is
+//               (src/models/qwen35/decoder.cpp:493,504-509; RmsNorm is
 //               src/core/vec.hpp:56-63).  Workgroup 0 also stores x + delta and the
 //               normalized row for the steps that follow.
 constexpr int kInPlain = kProloguePlain;
@@ -737,11 +737,12 @@ struct LdsX {
 // visited by one wave; this wave takes groups g_first, g_first + g_stride, ... below
 // g_end.  part_shift is added to every part's row pointer: the byte offset of an
 // expert inside its 3-D tensor (the parts of one launch share the expert stride).
-template <int TYPE, int NTOK, int kIn>
+// With kPick no output is stored: best[t] collects this lane's best output of column t.
+template <int TYPE, int NTOK, int kIn, bool kPick = false>
 __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NTOK>& col,
                                          const GemvPrologue& in, size_t part_shift,
                                          uint32_t g_first, uint32_t g_stride, uint32_t g_end,
-                                         U32x4* lds) {
+                                         U32x4* lds, Best* best = nullptr) {
   using Raw = typename RawOf<TYPE>::Type;
   using X = typename XOf<TYPE>::Type;
   constexpr int kBlockBytes = BlockBytes(TYPE);
@@ -867,7 +868,11 @@ __device__ __forceinline__ void GemvBody(const GemvParams& prm, const Columns<NT
         for (int t = 0; t < NTOK; ++t) {
           const float total = GroupTotal(acc[d][t], lanes_per_row);
           if (valid[d] && (lane & (lanes_per_row - 1)) == lanes_per_row - 1) {
-            col.y[t][y_index[d]] = total;
+            if (kPick) {
+              best[t] = Better(best[t], Best{total, y_index[d]});
+            } else {
+              col.y[t][y_index[d]] = total;
+            }
           }
         }
         locate(d, next_group0 + d * g_stride);
@@ -898,6 +903,75 @@ __attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(NTOK)))) void KquantGemvKerne
   const uint32_t wave = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
   GemvBody<TYPE, NTOK, kIn>(prm, col, in, 0, wave, gridDim.x * kWavesPerGroup, prm.n_groups,
                             lds);
+}
+
+// The dense product with the greedy pick inside: no y.  Every lane keeps the best output
+// it formed per token; the workgroup's best goes to pick.partial[t][blockIdx.x], and
+// GemvPickFinalKernel, launched behind it, takes the best of those (at most 768 per
+// token).  Better is a total order, so the result does not depend on how the rows were
+// spread over lanes and workgroups.  (Finishing inside this kernel - the last workgroup
+// to arrive, found with a device-scope counter, reduces - was built and measured: the
+// device-scope fences it needs around the counter made the 151,936-row head 77 us
+// against 50 us, as each fence writes back and invalidates an L2 that is per XCD.)
+template <int TYPE, int NTOK, int kIn>
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(WavesPerSimdFor(NTOK)))) void KquantGemvPickKernel(
+    const GemvParams prm, const GemvPrologue in, const float* __restrict__ x,
+    const GemvPick pick) {
+  extern __shared__ __align__(16) U32x4 lds[];
+  Columns<NTOK> col;
+#pragma unroll
+  for (int t = 0; t < NTOK; ++t) {
+    col.x[t] = x + static_cast<size_t>(t) * prm.cols;
+    col.y[t] = nullptr;
+  }
+  Best best[NTOK];
+#pragma unroll
+  for (int t = 0; t < NTOK; ++t) best[t] = Best{-INFINITY, kNoIndex};
+  const uint32_t wave = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  GemvBody<TYPE, NTOK, kIn, true>(prm, col, in, 0, wave, gridDim.x * kWavesPerGroup,
+                                  prm.n_groups, lds, best);
+
+  // The staged activations are dead once every wave has left the loop; their LDS now
+  // carries the wave results (NTOK x 4 candidates).
+  __syncthreads();
+  Best* wave_best = reinterpret_cast<Best*>(lds);
+#pragma unroll
+  for (int t = 0; t < NTOK; ++t) {
+    const Best of_wave = WaveBest(best[t]);
+    if ((threadIdx.x & 63) == 0) wave_best[t * kWavesPerGroup + (threadIdx.x >> 6)] = of_wave;
+  }
+  __syncthreads();
+  Best* partial = static_cast<Best*>(pick.partial);
+  if (threadIdx.x < NTOK) {
+    Best of_group = wave_best[threadIdx.x * kWavesPerGroup];
+#pragma unroll
+    for (int w = 1; w < kWavesPerGroup; ++w) {
+      of_group = Better(of_group, wave_best[threadIdx.x * kWavesPerGroup + w]);
+    }
+    partial[threadIdx.x * gridDim.x + blockIdx.x] = of_group;
+  }
+}
+
+// The best of the `groups` candidates of token blockIdx.x -> pick.index / pick.value.
+__global__ __launch_bounds__(kThreads) void GemvPickFinalKernel(const GemvPick pick,
+                                                                uint32_t groups) {
+  __shared__ Best wave_best[kWavesPerGroup];
+  const uint32_t t = blockIdx.x;
+  const Best* partial = static_cast<const Best*>(pick.partial) + t * groups;
+  Best mine{-INFINITY, kNoIndex};
+  for (uint32_t i = threadIdx.x; i < groups; i += kThreads) mine = Better(mine, partial[i]);
+  mine = WaveBest(mine);
+  if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best all = wave_best[0];
+#pragma unroll
+    for (int w = 1; w < kWavesPerGroup; ++w) all = Better(all, wave_best[w]);
+    // Nothing but -inf and NaN: max_element returns the first element.
+    pick.index[t] = all.index == kNoIndex ? 0 : static_cast<int64_t>(all.index);
+    if (pick.value != nullptr) pick.value[t] = all.value;
+  }
 }
 
 // Expert product: blockIdx.y names a segment, i.e. one routed expert and up to four
@@ -1039,6 +1113,35 @@ hipError_t LaunchTyped(const DenseCall& call, int tokens) {
   }
 }
 
+template <int TYPE, int NTOK, int kIn>
+hipError_t LaunchPick(const DenseCall& call, const GemvPick& pick) {
+  const hipError_t status =
+      AllowLargeLds(KquantGemvPickKernel<TYPE, NTOK, kIn>, call.lds_bytes);
+  if (status != hipSuccess) return status;
+  hipLaunchKernelGGL((KquantGemvPickKernel<TYPE, NTOK, kIn>), call.grid, dim3(kThreads),
+                     call.lds_bytes, call.stream, call.prm, call.in, call.x, pick);
+  hipLaunchKernelGGL(GemvPickFinalKernel, dim3(NTOK), dim3(kThreads), 0, call.stream, pick,
+                     call.grid.x);
+  return hipGetLastError();
+}
+
+template <int TYPE, int NTOK>
+hipError_t LaunchPickColumns(const DenseCall& call, const GemvPick& pick) {
+  return call.in.kind == kInResNorm ? LaunchPick<TYPE, NTOK, kInResNorm>(call, pick)
+                                    : LaunchPick<TYPE, NTOK, kInPlain>(call, pick);
+}
+
+template <int TYPE>
+hipError_t LaunchPickTyped(const DenseCall& call, const GemvPick& pick, int tokens) {
+  switch (tokens) {
+    case 1: return LaunchPickColumns<TYPE, 1>(call, pick);
+    case 2: return LaunchPickColumns<TYPE, 2>(call, pick);
+    case 3: return LaunchPickColumns<TYPE, 3>(call, pick);
+    case 4: return LaunchPickColumns<TYPE, 4>(call, pick);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int TYPE, bool kSwiGlu, int kMaxTok>
 hipError_t LaunchMoeKernel(const GemvParams& prm, const MoeGemvArgs& moe, dim3 grid,
                            size_t lds_bytes, hipStream_t stream) {
@@ -1082,6 +1185,60 @@ hipError_t LaunchGemv(int type, const GemvLaunch& launch, const float* x, int to
   return LaunchGemvFused(type, launch, GemvPrologue{}, x, tokens, y, stream);
 }
 
+namespace {
+
+// Checks a dense launch and fills everything of `call` but its output.
+hipError_t PlanDense(int type, const GemvLaunch& launch, const GemvPrologue& in,
+                     const float* x, int tokens, hipStream_t stream, DenseCall* call) {
+  if (!ValidLaunch(type, launch) || tokens < 1 ||
+      tokens > GemvMaxTokens(type, launch.blocks_per_row)) {
+    return hipErrorInvalidValue;
+  }
+  if (in.kind == kInResNorm && in.norm_weight == nullptr) return hipErrorInvalidValue;
+  call->in = in;
+  call->x = x;
+  call->y = nullptr;
+  call->stream = stream;
+  // kInResNorm keeps the four wave sums of every token behind the staged rows.
+  call->lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens) +
+                    (in.kind == kInResNorm ? kMaxGemvTokens * kWavesPerGroup * sizeof(float) : 0);
+  if (call->lds_bytes > kGemvMaxLdsBytes) return hipErrorInvalidValue;
+  PlanGemv(type, launch, &call->prm);
+  uint32_t blocks = (call->prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
+  // Persistent: no more workgroups than are resident at once.
+  const uint32_t resident =
+      static_cast<uint32_t>(g_compute_units) * WavesPerSimdFor(tokens);
+  if (blocks > resident) blocks = resident;
+  call->grid = dim3(blocks);
+  return hipSuccess;
+}
+
+}  // namespace
+
+size_t GemvPickPartialBytes(int tokens) {
+  return static_cast<size_t>(tokens > 0 ? tokens : 0) * g_compute_units *
+         WavesPerSimdFor(1) * sizeof(Best);
+}
+
+hipError_t LaunchGemvPick(int type, const GemvLaunch& launch, const GemvPrologue& in,
+                          const float* x, int tokens, const GemvPick& pick,
+                          hipStream_t stream) {
+  if (in.kind != kInPlain && in.kind != kInResNorm) return hipErrorInvalidValue;
+  if (pick.partial == nullptr || pick.index == nullptr || launch.total_rows == 0) {
+    return hipErrorInvalidValue;
+  }
+  DenseCall call;
+  const hipError_t status = PlanDense(type, launch, in, x, tokens, stream, &call);
+  if (status != hipSuccess) return status;
+  switch (type) {
+    case kTypeQ4K: return LaunchPickTyped<kTypeQ4K>(call, pick, tokens);
+    case kTypeQ5K: return LaunchPickTyped<kTypeQ5K>(call, pick, tokens);
+    case kTypeQ6K: return LaunchPickTyped<kTypeQ6K>(call, pick, tokens);
+    case kTypeQ80: return LaunchPickTyped<kTypeQ80>(call, pick, tokens);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 hipError_t LaunchGemvFused(int type, const GemvLaunch& launch, const GemvPrologue& in,
                            const float* x, int tokens, float* y, hipStream_t stream) {
   if (type == kTypeF32) {
@@ -1089,28 +1246,11 @@ hipError_t LaunchGemvFused(int type, const GemvLaunch& launch, const GemvPrologu
     if (in.kind != kInPlain) return hipErrorInvalidValue;
     return LaunchGemvF32(launch, x, tokens, y, stream);
   }
-  if (!ValidLaunch(type, launch) || tokens < 1 ||
-      tokens > GemvMaxTokens(type, launch.blocks_per_row)) {
-    return hipErrorInvalidValue;
-  }
-  if (in.kind == kInResNorm && in.norm_weight == nullptr) return hipErrorInvalidValue;
   DenseCall call;
-  call.in = in;
-  call.x = x;
-  call.y = y;
-  call.stream = stream;
-  // kInResNorm keeps the four wave sums of every token behind the staged rows.
-  call.lds_bytes = LdsBytes(type, launch.blocks_per_row, tokens) +
-                   (in.kind == kInResNorm ? kMaxGemvTokens * kWavesPerGroup * sizeof(float) : 0);
-  if (call.lds_bytes > kGemvMaxLdsBytes) return hipErrorInvalidValue;
+  const hipError_t status = PlanDense(type, launch, in, x, tokens, stream, &call);
+  if (status != hipSuccess) return status;
   if (launch.total_rows == 0) return hipSuccess;
-  PlanGemv(type, launch, &call.prm);
-  uint32_t blocks = (call.prm.n_groups + kWavesPerGroup - 1) / kWavesPerGroup;
-  // Persistent: no more workgroups than are resident at once.
-  const uint32_t resident =
-      static_cast<uint32_t>(g_compute_units) * WavesPerSimdFor(tokens);
-  if (blocks > resident) blocks = resident;
-  call.grid = dim3(blocks);
+  call.y = y;
   switch (type) {
     case kTypeQ4K: return LaunchTyped<kTypeQ4K>(call, tokens);
     case kTypeQ5K: return LaunchTyped<kTypeQ5K>(call, tokens);

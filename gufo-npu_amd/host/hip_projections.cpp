@@ -191,25 +191,14 @@ void HipProjections::Apply(Stage stage, int layer, const float* x, int tokens, f
                       x, tokens, y));
 }
 
-void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
-                                 float* y) const {
-  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
-  if (parts == nullptr || parts->empty()) {
-    throw std::logic_error("qwen35: no weights for this stage and layer");
-  }
-  std::vector<const gufo_hip_matrix*> handles;
-  std::vector<std::size_t> first;
-  std::vector<std::size_t> rows;
-  for (const Matrix& m : *parts) {
-    handles.push_back(m.handle);
-    first.push_back(0);
-    rows.push_back(m.rows);
-  }
+namespace {
+
+gufo_hip_prologue ToC(const HipProjections::DeviceInput& in) {
   gufo_hip_prologue prologue = {};
   switch (in.prologue) {
-    case Prologue::kPlain: prologue.kind = GUFO_HIP_PROLOGUE_PLAIN; break;
-    case Prologue::kSwiGlu: prologue.kind = GUFO_HIP_PROLOGUE_SWIGLU; break;
-    case Prologue::kResNorm:
+    case HipProjections::Prologue::kPlain: prologue.kind = GUFO_HIP_PROLOGUE_PLAIN; break;
+    case HipProjections::Prologue::kSwiGlu: prologue.kind = GUFO_HIP_PROLOGUE_SWIGLU; break;
+    case HipProjections::Prologue::kResNorm:
       prologue.kind = GUFO_HIP_PROLOGUE_RESNORM;
       prologue.delta_dev = in.delta;
       prologue.norm_weight_dev = in.norm_weight;
@@ -218,8 +207,51 @@ void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, 
       prologue.normed_out_dev = in.normed;
       break;
   }
-  Check(gufo_hip_gemv_fused_dev(handles.data(), first.data(), rows.data(),
-                                static_cast<int>(handles.size()), &prologue, in.x, tokens, y));
+  return prologue;
+}
+
+// The handles of a stage's matrices with their whole row ranges.
+struct WholeParts {
+  std::vector<const gufo_hip_matrix*> handles;
+  std::vector<std::size_t> first;
+  std::vector<std::size_t> rows;
+  int count() const { return static_cast<int>(handles.size()); }
+};
+
+}  // namespace
+
+void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
+                                 float* y) const {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  if (parts == nullptr || parts->empty()) {
+    throw std::logic_error("qwen35: no weights for this stage and layer");
+  }
+  WholeParts whole;
+  for (const Matrix& m : *parts) {
+    whole.handles.push_back(m.handle);
+    whole.first.push_back(0);
+    whole.rows.push_back(m.rows);
+  }
+  const gufo_hip_prologue prologue = ToC(in);
+  Check(gufo_hip_gemv_fused_dev(whole.handles.data(), whole.first.data(), whole.rows.data(),
+                                whole.count(), &prologue, in.x, tokens, y));
+}
+
+void HipProjections::PickDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
+                                std::int64_t* index) const {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  if (parts == nullptr || parts->empty()) {
+    throw std::logic_error("qwen35: no weights for this stage and layer");
+  }
+  WholeParts whole;
+  for (const Matrix& m : *parts) {
+    whole.handles.push_back(m.handle);
+    whole.first.push_back(0);
+    whole.rows.push_back(m.rows);
+  }
+  const gufo_hip_prologue prologue = ToC(in);
+  Check(gufo_hip_gemv_argmax_dev(whole.handles.data(), whole.first.data(), whole.rows.data(),
+                                 whole.count(), &prologue, in.x, tokens, index));
 }
 
 void HipProjections::ApplyExpert(Stage stage, int layer, int expert, const float* x, int tokens,

@@ -116,8 +116,8 @@ public:
   enum class Prologue {
     kPlain,    // x: tokens x StageInputs
     kSwiGlu,   // x: tokens x 2*StageInputs rows [gate | up] -> silu(gate) * up
-               // (decoder.cpp:509-512); the kFfnIn output feeds kFfnDown directly
-    kResNorm,  // RmsNorm(x + delta) * norm_weight (decoder.cpp:491,500-505); x + delta
+               // (decoder.cpp:511-514); the kFfnIn output feeds kFfnDown directly
+    kResNorm,  // RmsNorm(x + delta) * norm_weight (decoder.cpp:493,504-509); x + delta
                // goes to `residual`, the normalized rows to `normed` (either may be null)
   };
   struct DeviceInput {
@@ -130,6 +130,12 @@ public:
     float* normed = nullptr;
   };
   void ApplyDevice(Stage stage, int layer, const DeviceInput& in, int tokens, float* y) const;
+  // The stage's product with the greedy pick inside: index[t] (device memory) receives
+  // the position of the first maximum of the stage's output row for token t, which is
+  // never stored.  For Stage::kLmHead that is the greedy token (std::max_element over
+  // the logits, src/core/sampling.cpp:327-329).  kPlain and kResNorm inputs.
+  void PickDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
+                  std::int64_t* index) const;
 
   // qwen35::Route (src/models/qwen35/moe.cpp:16-42) on the device.
   void Route(const float* logits, int tokens, int k, int* chosen, float* weights) const;

@@ -11,6 +11,7 @@
 // bar is rel-L2 <= 1e-4 as for the kernels.
 #include <immintrin.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -367,7 +368,7 @@ private:
 };
 
 // The second half of a dense decoder layer on rows that stay on the device
-// (src/models/qwen35/decoder.cpp:500-512,526-528 of the reference): the residual add
+// (src/models/qwen35/decoder.cpp:504-515,519-521 of the reference): the residual add
 // and RmsNorm inside the kFfnIn product, SwiGLU inside the kFfnDown product - two
 // launches - against the same steps taken one at a time by the checker.
 void RunDeviceChain(std::mt19937& rng) {
@@ -442,6 +443,37 @@ void RunDeviceChain(std::mt19937& rng) {
          }));
 }
 
+// The greedy token straight from the head product: PickDevice against Apply followed by
+// std::max_element, with and without the output norm in front.
+void RunPick(std::mt19937& rng) {
+  const std::size_t hidden = 512, vocab = 3000;
+  const Weights head = RandomWeights(GUFO_ORACLE_Q6_K, vocab, hidden, rng);
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  model.lm_head = AsTensor("token_embd.weight", head);
+  const HipProjections proj(model);
+  for (const int tokens : {1, 4}) {
+    const auto n = static_cast<std::size_t>(tokens);
+    const auto x = RandomActivations(n * hidden, rng);
+    std::vector<float> logits(n * vocab);
+    proj.Apply(Stage::kLmHead, -1, x.data(), tokens, logits.data());
+    const DeviceRows d_x(x), d_index(2 * n);  // 2 floats = one int64 per token
+    HipProjections::DeviceInput in;
+    in.x = d_x.get();
+    proj.PickDevice(Stage::kLmHead, -1, in, tokens, reinterpret_cast<std::int64_t*>(d_index.get()));
+    const auto raw = d_index.Download();
+    bool same = true;
+    for (std::size_t t = 0; t < n; ++t) {
+      std::int64_t got;
+      std::memcpy(&got, &raw[2 * t], sizeof got);
+      const float* row = &logits[t * vocab];
+      same = same && got == std::max_element(row, row + vocab) - row;
+    }
+    Report("PickDevice kLmHead equals max_element of Apply tokens=" + std::to_string(tokens),
+           same);
+  }
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -451,6 +483,7 @@ int main(int argc, char** argv) {
     RunDense(rng);
     RunMoe(rng);
     RunDeviceChain(rng);
+    RunPick(rng);
   } catch (const std::exception& e) {
     std::fprintf(stderr, "FAIL: unexpected exception: %s\n", e.what());
     return 1;

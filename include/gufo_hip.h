@@ -141,18 +141,18 @@ int gufo_hip_gemv_dev(const gufo_hip_matrix* const* parts, const size_t* first_r
 
 /* What a product does to its activation rows before multiplying: the elementwise
  * steps Decoder::Step runs on the host between its products
- * (src/models/qwen35/decoder.cpp:491-512), taken into the product's own kernel the way
+ * (src/models/qwen35/decoder.cpp:493-521), taken into the product's own kernel the way
  * the reference's NPU GEMV takes them as input stages (Prologue,
  * src/npu/gemv.hpp:58-63), so that a decoder layer is four launches with nothing
  * between them.
  *   PLAIN    x[t] as given (cols values).
  *   SWIGLU   x[t] holds [gate | up], 2*cols values, e.g. the y row of the product
  *            before; the activation is silu(gate[i]) * up[i]
- *            (decoder.cpp:509-512, Silu at :28-33; here x / (1 + exp(-x)) in fp32).
+ *            (decoder.cpp:511-514, Silu at :28-33; here x / (1 + exp(-x)) in fp32).
  *   RESNORM  the activation is RmsNorm(x[t] + delta[t]) * norm_weight, with
  *            RmsNorm(v)[i] = v[i] * (1 / sqrt(mean(v^2) + eps)) * w[i] in fp32
  *            (src/core/vec.hpp:56-63): the residual add that ends one half of a layer
- *            (decoder.cpp:500-502,526-528) and the norm that opens the next (:491,505).
+ *            (decoder.cpp:504-506,519-521) and the norm that opens the next (:493,508).
  *            delta_dev may be NULL (the first layer has nothing to add).  If not NULL,
  *            residual_out_dev receives x + delta (the new residual stream) and
  *            normed_out_dev the normalized rows (for the router and the experts of a
@@ -179,6 +179,29 @@ int gufo_hip_gemv_fused_dev(const gufo_hip_matrix* const* parts, const size_t* f
                             const size_t* n_rows, int n_parts,
                             const gufo_hip_prologue* prologue, const float* x_dev,
                             int tokens, float* y_dev);
+
+/* The product with the greedy pick inside: index_dev[t] = position, within the
+ * concatenated output row, of the first maximum of y[t] (std::max_element's rule,
+ * src/core/sampling.cpp:327-329); y itself is never stored.  This is how the reference's
+ * NPU decoder reads its draft head (src/models/qwen36_35b_a3b/npu_decoder.cpp:968-973):
+ * a head product whose only consumer is max_element.  PLAIN and RESNORM prologues
+ * (RESNORM: the output norm in front of the head, decoder.cpp:525-526).  Enqueued only;
+ * index_dev is device memory (tokens x int64).  The pick rides inside the product's
+ * kernel (each workgroup keeps its best candidate; a small kernel behind it takes the
+ * best of those) when the product is one launch (quantized rows of one type,
+ * tokens <= 4); otherwise the product goes to library scratch and gufo_hip_argmax_dev's
+ * kernels pick. */
+int gufo_hip_gemv_argmax_dev(const gufo_hip_matrix* const* parts, const size_t* first_row,
+                             const size_t* n_rows, int n_parts,
+                             const gufo_hip_prologue* prologue, const float* x_dev,
+                             int tokens, int64_t* index_dev);
+
+/* A new matrix holding rows rows_host[0..n) of `src`, in that order: the draft
+ * vocabulary's rows of the head (qwen35::DraftVocab, src/models/qwen35/draft_vocab.hpp:7-14;
+ * q4nx::PackRows in npu_decoder.cpp:532-544).  A pick over it returns a position i; the
+ * token is rows_host[i].  Rows out of range: OUT_OF_RANGE. */
+int gufo_hip_matrix_gather_rows(const gufo_hip_matrix* src, const int64_t* rows_host,
+                                size_t n, gufo_hip_matrix** out);
 
 /* Greedy pick over logits, std::max_element's rule: the first maximum wins
  * (src/core/sampling.cpp:327-329).  `index` receives the position. */

@@ -133,13 +133,13 @@ void gufo_oracle_rms_norm(const float* x, const float* w, size_t n, float eps,
                           float* out);
 
 /* The residual add that ends a half layer and the norm that opens the next
- * (models/qwen35/decoder.cpp:500-505): residual = x + delta (delta NULL: x),
+ * (models/qwen35/decoder.cpp:504-509): residual = x + delta (delta NULL: x),
  * normed = RmsNorm(residual) * w.  residual may be NULL. */
 void gufo_oracle_res_norm(const float* x, const float* delta, const float* w, size_t n,
                           float eps, float* residual, float* normed);
 
 /* The activation between the two products of the dense feed-forward block
- * (models/qwen35/decoder.cpp:509-512 with Silu of :28-33, x * (1 / (1 + e^-x))):
+ * (models/qwen35/decoder.cpp:511-514 with Silu of :28-33, x * (1 / (1 + e^-x))):
  * act[i] = silu(gate_up[i]) * gate_up[f + i], i < f. */
 void gufo_oracle_swiglu(const float* gate_up, size_t f, float* act);
 

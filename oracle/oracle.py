@@ -266,7 +266,7 @@ def rms_norm(x: np.ndarray, w: np.ndarray, eps: float, use_ref: bool = False) ->
 
 def res_norm(x: np.ndarray, delta, w: np.ndarray, eps: float):
     """(residual, normed) of tokens x n rows: residual = x + delta, normed = RmsNorm(residual)
-    (models/qwen35/decoder.cpp:500-505).  delta may be None."""
+    (models/qwen35/decoder.cpp:504-509).  delta may be None."""
     x = np.atleast_2d(_f32(x))
     w = _f32(w)
     d = None if delta is None else np.atleast_2d(_f32(delta))
@@ -279,7 +279,7 @@ def res_norm(x: np.ndarray, delta, w: np.ndarray, eps: float):
 
 
 def swiglu(gate_up: np.ndarray) -> np.ndarray:
-    """silu(gate) * up of tokens x 2f rows [gate | up] (models/qwen35/decoder.cpp:509-512)."""
+    """silu(gate) * up of tokens x 2f rows [gate | up] (models/qwen35/decoder.cpp:511-514)."""
     g = np.atleast_2d(_f32(gate_up))
     f = g.shape[1] // 2
     act = np.empty((g.shape[0], f), dtype=np.float32)

@@ -220,7 +220,7 @@ def test_swiglu_product_parity(hip, oracle, ggml_type, rows, f):
 
 def test_decoder_layer_chain(hip, oracle):
     # The products of one dense layer as Decoder::Step orders them
-    # (src/models/qwen35/decoder.cpp:489-528 of the reference), with a stand-in for the
+    # (src/models/qwen35/decoder.cpp:491-521 of the reference), with a stand-in for the
     # mixer (it is not on this path): four launches, nothing between them, against the
     # same steps run one by one on the host.
     hidden, ffn = 2048, 6144  # the decode set's layer widths
