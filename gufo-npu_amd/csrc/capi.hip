@@ -1034,7 +1034,7 @@ int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* 
   if (m > (1ull << 24)) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens exceed the launch limit", m);
   }
-  GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmWorkspaceBytes(m, nb)));
+  GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmWorkspaceBytes(m, static_cast<uint32_t>(w->rows), nb)));
   GUFO_HIP_TRY(gufo::LaunchGemmQ4K(w->data, static_cast<uint32_t>(w->rows), nb, a, m,
                                    g_state.gemm_work.ptr, c, g_state.stream));
   return GUFO_HIP_OK;

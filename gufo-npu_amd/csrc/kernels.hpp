@@ -166,8 +166,8 @@ hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const
 
 // ---- prefill ------------------------------------------------------------------
 
-// Bytes of device workspace LaunchGemmQ4K needs for `tokens` activation rows.
-size_t GemmWorkspaceBytes(size_t tokens, uint32_t blocks_per_row);
+// Bytes of device workspace LaunchGemmQ4K needs: both operands as fp16.
+size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row);
 
 // c[t*rows + r] = row r of the Q4_K matrix w . a[t], a given as bf16 (tokens x
 // blocks_per_row*256), on the matrix cores with fp32 accumulation.

@@ -3,16 +3,15 @@
 // tokens = m (src/models/qwen35/gguf_projections.cpp:239-286 of the reference), the
 // shape the reference's NPU serves with its prefill GEMM (src/npu/gemm.hpp:99-105).
 //
-// The weights are dequantized in the kernel, in registers, to 16-bit operands and
-// never written to memory:
+// Two launches.  A pre-pass turns both operands into fp16 once per call; the product
+// kernel then only moves 16-bit operands and issues matrix instructions.
 //
 //   weight[r][k] = d * sc_j * q - dmin * m_j          (j = sub-block of k)
 //
 //   * 16-bit means fp16, not bf16: rounding the dequantized weight to bf16 (8-bit
 //     significand) costs 1.7e-3 relative L2 on this workload, above the 1e-3 this
 //     kernel is held to; fp16 (11 bits) costs 1.4e-4.  The bf16 activations convert
-//     to fp16 without loss (a pre-pass; magnitudes above 65504 saturate, below 2^-24
-//     flush).
+//     to fp16 without loss (magnitudes above 65504 saturate, below 2^-24 flush).
 //   * The 4-bit code becomes the fp16 number 1024 + q by a byte permute
 //     (0x6400 | q), and one fp32 fma with fp16 input and fp16 result
 //     (v_fma_mix) produces the weight with a single rounding:
@@ -20,26 +19,33 @@
 //     (11 x 6 bits); the offset is rounded to fp32 once per sub-block, 2^-14 of a
 //     quantization step.
 //   * v_mfma_f32_32x32x16_f16 accumulates in fp32 over the whole row.
+//   * Dequantizing once instead of inside the product kernel: with 4096 tokens every
+//     weight is used by 32 token tiles, and built in registers each time (the first
+//     version of this kernel) the conversion took as many issue cycles as the matrix
+//     instructions themselves: 124-133 us.  Written once as fp16 (25 MB for 6144 x 2048,
+//     5 us) the product kernel has no arithmetic left but the matrix instructions.
 //
 // Decomposition: one persistent workgroup of 8 waves per CU walks its share of the
-// 128-token x 256-row tiles.  Each wave owns 32 weight rows: it reads their packed
-// blocks into registers one super-block ahead, builds the operand fragments on the
-// fly and multiplies them with the four 32-token tiles.  The activations of half a
-// super-block (128 tokens x 128 fp16 = 32 KB, a "stage") go from global memory
-// straight into LDS (global_load_lds_dwordx4) into a ring of four stages, three
-// halves ahead of the matrix cores - across tile boundaries too, so the copies of a
-// tile's first halves and the stores of the previous tile's results overlap.
+// 128-token x 256-row tiles.  Each wave owns 32 weight rows and multiplies them with the
+// four 32-token tiles.  The activations of half a super-block (128 tokens x 128 fp16 =
+// 32 KB, a "stage") go from global memory straight into LDS (global_load_lds_dwordx4)
+// into a ring of four stages, three halves ahead of the matrix cores - across tile
+// boundaries too, so the copies of a tile's first halves and the stores of the previous
+// tile's results overlap.  The weight operand of a half (8 steps x 16 bytes per lane)
+// comes from the pre-pass's array straight into registers, one half ahead.
 //
 // The matrix instruction does not care which k a lane's 8 values belong to as long as
 // both operands agree, so k is dealt to lanes the way the packed block likes it: of
 // each 64 values (32 bytes of codes: low nibbles one sub-block, high nibbles the
 // next), lane half u owns bytes 16 u .. 16 u + 15 - one 16-byte load - and its four
-// steps take (low, first 8), (low, second 8), (high, first 8), (high, second 8).
+// steps take (low, first 8), (low, second 8), (high, first 8), (high, second 8).  The
+// pre-pass stores each (32 rows, super-block, step) as the 64 lanes' 16 bytes in lane
+// order, 1 KB, so the product kernel's loads are whole cache lines.
 //
 // Tiles are ordered (band of row tiles, token tile, row tile within the band) and the
 // order is cut in 8 pieces, one per XCD (workgroups go to XCDs round-robin): an XCD's
-// slice of the packed matrix stays in its L2 while it walks the token tiles, and the
-// workgroups running together share activation tiles.
+// slice of the fp16 matrix (3 of the 24 row tiles, 3 MB) stays in its L2 while it walks
+// the token tiles, and the workgroups running together share activation tiles.
 #include <type_traits>
 
 #include "kernels.hpp"
@@ -59,93 +65,15 @@ constexpr int kTileTokens = 128;
 constexpr int kTileRows = 32 * kGemmWaves;
 constexpr int kRowBytes = 256;                            // one token's half super-block as fp16
 constexpr int kStageBytes = kTileTokens * kRowBytes;      // 32 KB
-constexpr int kStages = 4;
-constexpr int kAhead = kStages - 1;                       // halves the copies run ahead
+constexpr int kStages = 4;                                // the copies run kStages - 1 halves ahead
 constexpr int kCopiesPerWave = kStageBytes / 1024 / kGemmWaves;  // 1 KB per wave instruction
-constexpr int kRowLoads = 5;                              // vector loads of one PackedRow
-constexpr int kTileStores = 16;                           // 16-byte stores of a whole tile, per wave
-// Operations a wave has issued after the copies of half h when it reaches the top of
-// half h: the copies of two more halves and the row loads of one (h even) or two blocks.
-constexpr int kEvenYounger = 2 * kCopiesPerWave + kRowLoads;
-constexpr int kOddYounger = 2 * kCopiesPerWave + 2 * kRowLoads;
+constexpr int kStepsPerHalf = 8;
+constexpr int kStepBytes = 64 * 16;                       // one step's fragments of 32 rows
+constexpr int kHalfBytes = kStepsPerHalf * kStepBytes;    // 8 KB per 32 rows and half super-block
 constexpr int kQ4Block = 144;
 constexpr int kXcds = 8;
 
-// ---- pre-pass: bf16 activations -> fp16, same [token][k] layout -------------------
-__global__ __launch_bounds__(256) void PrepareActivations(const U32x4* __restrict__ a,
-                                                          size_t octets,
-                                                          U32x4* __restrict__ out) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (i >= octets) return;
-  const U32x4 raw = a[i];
-  const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
-  uint32_t packed[4];
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    float lo = __uint_as_float(in[p] << 16);
-    float hi = __uint_as_float(in[p] & 0xFFFF0000u);
-    lo = __builtin_fminf(__builtin_fmaxf(lo, -65504.0f), 65504.0f);
-    hi = __builtin_fminf(__builtin_fmaxf(hi, -65504.0f), 65504.0f);
-    const Half2 h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
-    packed[p] = __builtin_bit_cast(uint32_t, h);
-  }
-  out[i] = U32x4{packed[0], packed[1], packed[2], packed[3]};
-}
-
-// ---- the product ------------------------------------------------------------------
-
-// Where the 16-byte piece p (0..15) of token row t sits inside the row's 256 bytes of
-// LDS: slot p ^ Swizzle(t).  Rows are one bank sweep apart, so the slot alone decides
-// the banks; a wave reads piece (c | 2 u) of rows n = 0..31, and the xor makes the 16
-// slots of rows n..n+15 (either u) and of rows n..n+7 (both u) all different.
-__device__ __forceinline__ uint32_t Swizzle(uint32_t t) {
-  return (t & 1u) | (((t >> 1) & 3u) << 2) | (((t >> 3) & 1u) << 1);
-}
-
-// One weight row's packed super-block as this lane reads it: lane (n, u) = (lane % 32,
-// lane / 32) takes bytes 16 u .. 16 u + 15 of each 32 bytes of codes of row n.
-//
-// The loads are issued from inline assembly and waited for by WaitForRow below, not by
-// the compiler: its own bookkeeping falls back to draining every vector-memory
-// operation - the copies into LDS that are meant to stay in flight included - once the
-// stores of a finished tile are pending in the same loop.
-struct PackedRow {
-  U32x4 header;     // d, dmin, 12 scale bytes
-  U32x4 codes[4];   // codes[p] = qs[32 p + 16 u .. +16)
-
-  // Starts the kRowLoads loads; the fields hold nothing until WaitForRow has returned.
-  __device__ __forceinline__ void StartLoad(const uint8_t* blk, uint32_t u) {
-    const uint8_t* half = blk + 16 * u;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(header) : "v"(blk) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(codes[0]) : "v"(half) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:48" : "=v"(codes[1]) : "v"(half) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:80" : "=v"(codes[2]) : "v"(half) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:112" : "=v"(codes[3]) : "v"(half) : "memory");
-  }
-};
-
-// Waits until at most kYounger vector-memory operations issued after row's loads are
-// outstanding, which is when the loads have landed; ties the fields to the wait so that
-// no use of them moves above it.
-template <int kYounger>
-__device__ __forceinline__ void WaitForRow(PackedRow& row) {
-  static_assert(kYounger == 0 || kYounger == kCopiesPerWave,
-                "the counts the copy schedule produces");
-  static_assert(kCopiesPerWave == 4, "update the literal below");
-  if constexpr (kYounger == 0) {
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(row.header), "+v"(row.codes[0]), "+v"(row.codes[1]), "+v"(row.codes[2]),
-                   "+v"(row.codes[3])
-                 :
-                 : "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(4)"
-                 : "+v"(row.header), "+v"(row.codes[0]), "+v"(row.codes[1]), "+v"(row.codes[2]),
-                   "+v"(row.codes[3])
-                 :
-                 : "memory");
-  }
-}
+// ---- pre-pass ---------------------------------------------------------------------
 
 // Two 4-bit codes (bytes of `nibbles` picked by `selector`, each 0..15) dequantized to
 // two fp16: the permute builds 0x6400 | q = 1024 + q, the fma runs in fp32.
@@ -170,15 +98,15 @@ __device__ __forceinline__ void SubBlockAffine(const U32x4& header, int j, float
   *offset = __builtin_fmaf(-dmin, static_cast<float>(mn), -1024.0f * *scale);
 }
 
-// Step s = 4 p + 2 high + half of a super-block: this lane's 8 dequantized values,
-// k = 64 p + 32 high + 16 u + 8 half .. +8 of sub-block j = 2 p + high = s / 2, whose
-// scale and offset the caller passes.
-__device__ __forceinline__ Half8 WeightFragment(const PackedRow& row, int s, float scale,
+// Step s = 4 p + q, q = 2 high + half, of a super-block: this lane's 8 dequantized
+// values, k = 64 p + 32 high + 16 u + 8 half .. +8, of sub-block j = 2 p + high, whose
+// scale and offset the caller passes.  `codes` = qs[32 p + 16 u .. +16): the lane's 16
+// bytes of the 64 values 64 p .. 64 p + 63.
+__device__ __forceinline__ U32x4 WeightFragment(const U32x4& codes, int q, float scale,
                                                 float offset) {
-  const int p = s >> 2;
-  const uint32_t b0 = (s & 1) ? row.codes[p].z : row.codes[p].x;
-  const uint32_t b1 = (s & 1) ? row.codes[p].w : row.codes[p].y;
-  const uint32_t shift = (s & 2) ? 4 : 0;
+  const uint32_t b0 = (q & 1) ? codes.z : codes.x;
+  const uint32_t b1 = (q & 1) ? codes.w : codes.y;
+  const uint32_t shift = (q & 2) ? 4 : 0;
   const uint32_t n0 = (b0 >> shift) & 0x0F0F0F0Fu;
   const uint32_t n1 = (b1 >> shift) & 0x0F0F0F0Fu;
   // perm selectors: result bytes [3..0] = [0x64, q_hi, 0x64, q_lo]; source 1 (nibbles)
@@ -188,7 +116,164 @@ __device__ __forceinline__ Half8 WeightFragment(const PackedRow& row, int s, flo
   out.y = DequantPair(n0, 0x04030402u, scale, offset);  // codes 2, 3
   out.z = DequantPair(n1, 0x04010400u, scale, offset);  // codes 4, 5
   out.w = DequantPair(n1, 0x04030402u, scale, offset);  // codes 6, 7
-  return __builtin_bit_cast(Half8, out);
+  return out;
+}
+
+// Both operands as fp16, one launch.  Every wave of workgroups [0, weight_groups)
+// dequantizes a quarter (64 values, 4 steps) of one super-block of one group of 32 rows
+// into fragments: w16[((group * nb + block) * 16 + step) * 64 + lane] (16 bytes each);
+// rows past the matrix repeat its last row, their products are not stored.  The other
+// workgroups convert 256 octets of activations each (bf16 -> fp16, same [token][k]
+// layout).
+__global__ __launch_bounds__(256) void PrepareOperands(
+    const U32x4* __restrict__ a, size_t octets, U32x4* __restrict__ a16,
+    uint32_t weight_groups, const uint8_t* __restrict__ w, uint32_t rows, uint32_t nb,
+    uint32_t row_groups, U32x4* __restrict__ w16) {
+  if (blockIdx.x >= weight_groups) {
+    const size_t i = static_cast<size_t>(blockIdx.x - weight_groups) * 256 + threadIdx.x;
+    if (i >= octets) return;
+    const U32x4 raw = a[i];
+    const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t packed[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      float lo = __uint_as_float(in[p] << 16);
+      float hi = __uint_as_float(in[p] & 0xFFFF0000u);
+      lo = __builtin_fminf(__builtin_fmaxf(lo, -65504.0f), 65504.0f);
+      hi = __builtin_fminf(__builtin_fmaxf(hi, -65504.0f), 65504.0f);
+      const Half2 h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+      packed[p] = __builtin_bit_cast(uint32_t, h);
+    }
+    a16[i] = U32x4{packed[0], packed[1], packed[2], packed[3]};
+    return;
+  }
+  const uint32_t quarter_unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t unit = quarter_unit >> 2;  // (group, block)
+  const uint32_t p = quarter_unit & 3;      // values 64 p .. 64 p + 63: steps 4 p .. 4 p + 3
+  if (unit >= row_groups * nb) return;
+  const uint32_t group = unit / nb;
+  const uint32_t block = unit - group * nb;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t n = lane & 31;
+  const uint32_t u = lane >> 5;
+  const uint32_t r = min(group * 32 + n, rows - 1);
+  const uint8_t* blk = w + (static_cast<size_t>(r) * nb + block) * kQ4Block;
+  const U32x4 header = Load16(blk);
+  const U32x4 codes = Load16(blk + 16 + 32 * p + 16 * u);
+  U32x4* out = w16 + (static_cast<size_t>(unit) * 16 + 4 * p) * 64 + lane;
+#pragma unroll
+  for (int high = 0; high < 2; ++high) {
+    float scale, offset;
+    SubBlockAffine(header, 2 * p + high, &scale, &offset);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      out[(2 * high + half) * 64] = WeightFragment(codes, 2 * high + half, scale, offset);
+    }
+  }
+}
+
+// ---- the product ------------------------------------------------------------------
+
+// Where the 16-byte piece p (0..15) of token row t sits inside the row's 256 bytes of
+// LDS: slot p ^ Swizzle(t).  Rows are one bank sweep apart, so the slot alone decides
+// the banks; a wave reads piece (c | 2 u) of rows n = 0..31, and the xor makes the 16
+// slots of rows n..n+15 (either u) and of rows n..n+7 (both u) all different.
+__device__ __forceinline__ uint32_t Swizzle(uint32_t t) {
+  return (t & 1u) | (((t >> 1) & 3u) << 2) | (((t >> 3) & 1u) << 1);
+}
+
+// This lane's weight operand of one half super-block: the fragments of its 8 steps.
+//
+// The loads are issued from inline assembly and waited for by WaitForFragments below, not
+// by the compiler: its own bookkeeping falls back to draining every vector-memory
+// operation - the copies into LDS that are meant to stay in flight included - once the
+// stores of a finished tile are pending in the same loop.
+struct Fragments {
+  U32x4 step[kStepsPerHalf];
+
+  // `at` is this lane's 16 bytes of step 0; the steps are kStepBytes apart.  The fields
+  // hold nothing until WaitForFragments has returned.
+  // The loads of steps 2 kPair and 2 kPair + 1 alone: the product kernel deals the eight
+  // loads of a half over the first four steps of the half before.
+  template <int kPair>
+  __device__ __forceinline__ void StartLoadPair(const uint8_t* at) {
+    static_assert(kPair >= 0 && kPair < 4, "four pairs of steps");
+    const uint8_t* base = at + (kPair / 2) * 4 * kStepBytes;
+    if constexpr (kPair % 2 == 0) {
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[2 * kPair]) : "v"(base) : "memory");
+      asm volatile("global_load_dwordx4 %0, %1, off offset:1024"
+                   : "=v"(step[2 * kPair + 1]) : "v"(base) : "memory");
+    } else {
+      asm volatile("global_load_dwordx4 %0, %1, off offset:2048"
+                   : "=v"(step[2 * kPair]) : "v"(base) : "memory");
+      asm volatile("global_load_dwordx4 %0, %1, off offset:3072"
+                   : "=v"(step[2 * kPair + 1]) : "v"(base) : "memory");
+    }
+  }
+
+  __device__ __forceinline__ void StartLoad(const uint8_t* at) {
+    const uint8_t* upper = at + 4 * kStepBytes;  // the offset field reaches 4 KB
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[0]) : "v"(at) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=v"(step[1]) : "v"(at) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=v"(step[2]) : "v"(at) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=v"(step[3]) : "v"(at) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[4]) : "v"(upper) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=v"(step[5]) : "v"(upper) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=v"(step[6]) : "v"(upper) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=v"(step[7]) : "v"(upper) : "memory");
+  }
+};
+static_assert(kStepBytes == 1024 && kStepsPerHalf == 8, "the offsets above");
+
+// Waits until f's loads have landed: until at most the kCopiesPerWave copies into LDS
+// that every StartLoad is followed by are outstanding (operations retire in order, loads,
+// copies and stores alike, so everything older has landed too).  Ties the fields to the
+// wait so that no use of them moves above it.
+__device__ __forceinline__ void WaitForFragments(Fragments& f) {
+  static_assert(kCopiesPerWave == 4, "update the literal below");
+  asm volatile("s_waitcnt vmcnt(4)"
+               : "+v"(f.step[0]), "+v"(f.step[1]), "+v"(f.step[2]), "+v"(f.step[3]),
+                 "+v"(f.step[4]), "+v"(f.step[5]), "+v"(f.step[6]), "+v"(f.step[7])
+               :
+               : "memory");
+}
+
+// The byte address inside LDS of a pointer into the stage ring.
+__device__ __forceinline__ uint32_t LdsAddress(const uint8_t* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((LdsPointer)p));
+}
+
+// This lane's activation operands of one step: its 16 bytes of the four 32-token tiles
+// (32 token rows = 8 KB apart).  Read and waited for from inline assembly for the same
+// reason as the weights: the wait is a count the compiler does not find.
+struct ActivationFragments {
+  U32x4 tile[4];
+
+  __device__ __forceinline__ void StartRead(uint32_t at) {
+    static_assert(32 * kRowBytes == 8192, "the offsets below");
+    asm volatile("ds_read_b128 %0, %1" : "=v"(tile[0]) : "v"(at) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(tile[1]) : "v"(at) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(tile[2]) : "v"(at) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:24576" : "=v"(tile[3]) : "v"(at) : "memory");
+  }
+};
+
+// Waits until at most kYounger LDS reads issued after f's are outstanding (LDS reads
+// return in order): 4 when the next step's reads follow, 0 for the last step of a half.
+template <int kYounger>
+__device__ __forceinline__ void WaitForActivations(ActivationFragments& f) {
+  static_assert(kYounger == 0 || kYounger == 4, "the counts the step loop produces");
+  if constexpr (kYounger == 0) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.tile[0]), "+v"(f.tile[1]), "+v"(f.tile[2]), "+v"(f.tile[3])
+                 :
+                 : "memory");
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(4)"
+                 : "+v"(f.tile[0]), "+v"(f.tile[1]), "+v"(f.tile[2]), "+v"(f.tile[3])
+                 :
+                 : "memory");
+  }
 }
 
 // The 16-byte piece of a token's half super-block that step s (0..7 within the half)
@@ -232,24 +317,6 @@ __device__ __forceinline__ TileCoord DecodeTile(const GemmShape& shape, uint32_t
   return tile;
 }
 
-// Waits until at most kPending of this wave's vector-memory operations are outstanding
-// (they retire in order, loads, copies into LDS and stores alike).
-template <int kPending>
-__device__ __forceinline__ void WaitVectorMemory() {
-  if constexpr (kPending == 0) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  } else if constexpr (kPending == 13) {
-    asm volatile("s_waitcnt vmcnt(13)" ::: "memory");
-  } else if constexpr (kPending == 18) {
-    asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-  } else if constexpr (kPending == 29) {
-    asm volatile("s_waitcnt vmcnt(29)" ::: "memory");
-  } else {
-    static_assert(kPending == 34, "a count the copy schedule does not produce");
-    asm volatile("s_waitcnt vmcnt(34)" ::: "memory");
-  }
-}
-
 // The workgroup barrier alone.  __syncthreads() adds a release fence that drains every
 // vector-memory operation of the wave, the prefetches included; here the waits that
 // matter are explicit: each wave waits for its own copies into LDS before the barrier,
@@ -262,15 +329,16 @@ __device__ __forceinline__ void TileBarrier() {
 // One workgroup per CU (the stage ring takes 128 KB of LDS): 2 waves per SIMD.
 //
 // The stream: this workgroup's tiles one after the other, each 2 nb halves.  Per wave,
-// vector-memory operations are issued in a fixed order - at the top of stream half h
-// the copies of half h + 3 (kCopiesPerWave instructions), then, if h is even, the
-// packed rows of the block after the current one (kRowLoads loads) - so that "the
-// copies of half h have landed" is a fixed count of younger operations allowed in
-// flight: 13 for even h, 18 for odd h.  Stores of finished tiles only add younger
-// operations, which makes a wait stricter, never too weak.  The last two blocks of
-// the stream, where copies run out, drain completely instead.
+// every half issues the same vector-memory operations in the same order - after the
+// barrier the stores of the tile the half before completed (if any), then the weight
+// fragments of half h + 1 (8 loads), then the copies of half h + 3 (kCopiesPerWave
+// instructions) - and, after its matrix instructions, waits until only those copies may
+// still be in flight: the fragments of half h + 1 have then landed, and with them
+// everything older, the copies of half h + 1 among it.  Past the end of the stream the
+// loads and copies repeat the last half into registers and a stage nobody uses, so the
+// count never changes.
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void
-KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
+KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a16,
                  float* __restrict__ c, GemmShape shape) {
   extern __shared__ __align__(1024) uint8_t stages[];  // kStages x kStageBytes
 
@@ -289,8 +357,7 @@ KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
   const uint32_t n = lane & 31;
   const uint32_t u = lane >> 5;
   const uint32_t nb = shape.nb;
-  const uint32_t total_blocks = n_tiles * nb;
-  const uint32_t total_halves = 2 * total_blocks;
+  const uint32_t total_halves = 2 * n_tiles * nb;
 
   // ---- copies global -> LDS ----
   // Wave instruction i of this wave fills the 1 KB holding token rows 4 c .. 4 c + 3 of
@@ -298,7 +365,9 @@ KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
   // 4 c + l / 16, that is piece slot ^ Swizzle(row) of the token's half block.  Rows
   // past the last token repeat it; their products are not stored.
   uint32_t copy_offset[kCopiesPerWave];  // bytes from a16 + 256 * (half within the tile)
-  auto aim_copies = [&](uint32_t token_tile) {
+  // (Every lambda below is inlined by force: one left as a call would take the
+  // accumulators and the fragments it captures by reference out of their registers.)
+  auto aim_copies = [&](uint32_t token_tile) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kCopiesPerWave; ++i) {
       const uint32_t t = 4 * (wave * kCopiesPerWave + i) + (lane >> 4);
@@ -306,45 +375,63 @@ KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
       copy_offset[i] = token * (nb * 512) + (((lane & 15u) ^ Swizzle(t & 15u)) << 4);
     }
   };
+  // Past the end of the stream the last half is copied again, into a stage nobody reads
+  // any more: every half issues the same operations, which keeps the wait a constant.
   uint32_t copy_half = 0;    // stream half the next copy brings in
   uint32_t copy_within = 0;  // the same, within its tile
   uint32_t copy_tile = 0;    // index into this workgroup's tiles
-  auto copy_next_half = [&]() {
+  struct CopyPlan {
+    const uint8_t* source[kCopiesPerWave];
+    uint8_t* stage;
+  };
+  // Where the copies of the next half read and write; moves on to the half after it.
+  auto plan_next_copy = [&]() __attribute__((always_inline)) {
+    CopyPlan plan;
     const uint8_t* base = a16 + static_cast<size_t>(copy_within) * kRowBytes;
-    uint8_t* stage = stages + (copy_half % kStages) * kStageBytes;
 #pragma unroll
-    for (int i = 0; i < kCopiesPerWave; ++i) {
-      uint8_t* dst = stage + (wave * kCopiesPerWave + i) * 1024;
-      __builtin_amdgcn_global_load_lds(base + copy_offset[i], (LdsPointer)dst, 16, 0, 0);
-    }
-    ++copy_half;
-    if (++copy_within == 2 * nb) {
+    for (int i = 0; i < kCopiesPerWave; ++i) plan.source[i] = base + copy_offset[i];
+    plan.stage = stages + (copy_half % kStages) * kStageBytes + wave * kCopiesPerWave * 1024;
+    if (++copy_half < total_halves && ++copy_within == 2 * nb) {
       copy_within = 0;
-      if (++copy_tile < n_tiles) {
-        aim_copies(DecodeTile(shape, first + copy_tile * stride).token_tile);
-      }
+      ++copy_tile;
+      aim_copies(DecodeTile(shape, first + copy_tile * stride).token_tile);
     }
+    return plan;
+  };
+  auto start_copy = [&](const CopyPlan& plan, int i) __attribute__((always_inline)) {
+    __builtin_amdgcn_global_load_lds(plan.source[i], (LdsPointer)(plan.stage + i * 1024), 16, 0, 0);
+  };
+  auto start_copies = [&](const CopyPlan& plan) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kCopiesPerWave; ++i) start_copy(plan, i);
   };
 
-  // ---- packed weight rows, one block ahead ----
-  const uint8_t* load_ptr = nullptr;  // this lane's row, next block to load
+  // ---- weight fragments, one half ahead ----
+  // Past the end of the stream the last half is loaded again and never used.
+  const uint8_t* load_ptr = nullptr;  // this lane's 16 bytes of step 0 of the next half to load
+  uint32_t load_half = 0;
   uint32_t load_within = 0;
   uint32_t load_tile = 0;
-  auto aim_loads = [&](uint32_t row_tile) {
-    const uint32_t r = min(row_tile * kTileRows + wave * 32 + n, shape.rows - 1);
-    load_ptr = w + static_cast<size_t>(r) * nb * kQ4Block;
+  auto aim_loads = [&](uint32_t row_tile) __attribute__((always_inline)) {
+    const size_t group = static_cast<size_t>(row_tile) * kGemmWaves + wave;
+    load_ptr = w16 + group * nb * 2 * kHalfBytes + lane * 16;
   };
-  auto load_next_block = [&](PackedRow& into) {
-    into.StartLoad(load_ptr, u);
-    load_ptr += kQ4Block;
-    if (++load_within == nb) {
-      load_within = 0;
-      if (++load_tile < n_tiles) aim_loads(DecodeTile(shape, first + load_tile * stride).row_tile);
+  // Where the fragments of the next half are; moves on to the half after it.
+  auto plan_next_load = [&]() __attribute__((always_inline)) {
+    const uint8_t* at = load_ptr;
+    if (++load_half < total_halves) {
+      load_ptr += kHalfBytes;
+      if (++load_within == 2 * nb) {
+        load_within = 0;
+        ++load_tile;
+        aim_loads(DecodeTile(shape, first + load_tile * stride).row_tile);
+      }
     }
+    return at;
   };
 
   Float16v acc[4];
-  auto clear_acc = [&]() {
+  auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
 #pragma unroll
@@ -358,76 +445,59 @@ KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
   const uint32_t flip = Swizzle(n & 15u) ^ (u << 1);
   const uint32_t read_base = n * kRowBytes;
 
-  // The weight operand runs one step ahead of the matrix cores across halves, blocks
-  // and tiles: `bf` enters a half holding its first step's fragment and leaves holding
-  // the next half's; `scale`/`offset` belong to the sub-block last dequantized.
-  Half8 bf;
-  float scale, offset;
-
   // One half super-block: 8 steps on the stage of stream half `half`.  While step s
-  // multiplies, the activation fragments of step s + 1 are on their way from LDS and
-  // the weight fragment of the step after it (of `follow`, the next block, after the
-  // last step of a block) is being dequantized between the matrix instructions.
-  // follow's loads are waited for just before that, with kYounger operations issued since.
-  auto multiply_half = [&](uint32_t half, const PackedRow& cur, PackedRow& follow, auto half_tag,
-                           auto younger_tag) {
-    constexpr int kHalf = decltype(half_tag)::value;
-    constexpr int kYounger = decltype(younger_tag)::value;
-    const uint8_t* tile = stages + (half % kStages) * kStageBytes + read_base;
-    Half8 af[4];
+  // multiplies, the activation fragments of step s + 1 are on their way from LDS: the
+  // reads of step s + 1 are issued, then the wait lets exactly those four stay in flight.
+  // (Left to the compiler the wait becomes lgkmcnt(0) on every second step, which puts a
+  // whole LDS latency in front of the matrix instructions: 55% of the waves' time.)
+  //
+  // The half's vector-memory operations ride along, behind the matrix instructions of
+  // the steps: the next half's weight fragments two loads a step over steps 0-3, the
+  // copies of the half three ahead one a step over steps 4-7.  Issued in one burst after
+  // the barrier - when all eight waves of the workgroup are at the same point - they
+  // queued up at the one address unit with no matrix instruction to cover them (measured:
+  // 46 of 115 us).
+  auto multiply_half = [&](uint32_t half, const Fragments& weights, Fragments& later,
+                           const uint8_t* later_at, const CopyPlan& copies)
+                           __attribute__((always_inline)) {
+    const uint32_t tile = LdsAddress(stages + (half % kStages) * kStageBytes + read_base);
+    ActivationFragments af[2];
+    af[0].StartRead(tile + ((StepPiece(0) ^ flip) << 4));
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      af[m] = *reinterpret_cast<const Half8*>(tile + ((StepPiece(0) ^ flip) << 4) +
-                                              m * 32 * kRowBytes);
-    }
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      Half8 af_next[4];
-      if (s + 1 < 8) {
-        const uint8_t* at = tile + ((StepPiece(s + 1) ^ flip) << 4);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          af_next[m] = *reinterpret_cast<const Half8*>(at + m * 32 * kRowBytes);
-        }
+    for (int s = 0; s < kStepsPerHalf; ++s) {
+      if (s + 1 < kStepsPerHalf) {
+        af[(s + 1) & 1].StartRead(tile + ((StepPiece(s + 1) ^ flip) << 4));
+        WaitForActivations<4>(af[s & 1]);
+      } else {
+        WaitForActivations<0>(af[s & 1]);
       }
-      // Nothing moves across: the reads of step s + 1 are issued before step s multiplies.
-      __builtin_amdgcn_sched_barrier(0);
-      const int upcoming = 8 * kHalf + s + 1;  // the step being dequantized
-      if (upcoming == 16) WaitForRow<kYounger>(follow);
-      const PackedRow& source = upcoming < 16 ? cur : follow;
-      if (upcoming % 2 == 0) {
-        SubBlockAffine(source.header, (upcoming % 16) / 2, &scale, &offset);
-      }
-      const Half8 bf_next = WeightFragment(source, upcoming % 16, scale, offset);
+      const Half8 bf = __builtin_bit_cast(Half8, weights.step[s]);
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af[m], acc[m], 0, 0, 0);
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            bf, __builtin_bit_cast(Half8, af[s & 1].tile[m]), acc[m], 0, 0, 0);
       }
-      // Within the step: each matrix instruction followed by a quarter of that work.
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
-      }
+      // The reads of step s + 2 reuse this step's registers: not before it has multiplied.
       __builtin_amdgcn_sched_barrier(0);
-      if (s + 1 < 8) {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) af[m] = af_next[m];
-      }
-      bf = bf_next;
+      if (s == 0) later.template StartLoadPair<0>(later_at);
+      if (s == 1) later.template StartLoadPair<1>(later_at);
+      if (s == 2) later.template StartLoadPair<2>(later_at);
+      if (s == 3) later.template StartLoadPair<3>(later_at);
+      if (s >= 4) start_copy(copies, s - 4);
+      __builtin_amdgcn_sched_barrier(0);  // the wait of the half counts on this issue order
     }
   };
 
   // ---- the tile being multiplied ----
   uint32_t tile_index = 0;
-  uint32_t block_within = 0;
+  uint32_t half_within = 0;
   TileCoord tile = DecodeTile(shape, first);
   // With the weights as the first operand, accumulator register i of token tile m holds
   // weight row 8 (i/4) + 4 u + i%4 of this wave's 32 and token 32 m + n: four registers
   // are four consecutive floats of a row of c.  A tile that lies wholly inside c stores
   // them as kTileStores 16-byte stores per wave; a ragged one stores float by float.
   // Returns whether the fixed number of stores was issued.
-  auto finish_tile = [&]() -> bool {
+  auto finish_tile = [&]() __attribute__((always_inline)) -> bool {
     const uint32_t row0 = tile.row_tile * kTileRows + wave * 32;
     const uint32_t token_first = tile.token_tile * kTileTokens;
     const bool whole = shape.vector_stores != 0 && row0 + 32 <= shape.rows &&
@@ -461,77 +531,57 @@ KquantGemmKernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ a16,
     return whole;
   };
 
+  // Stream half h on `now` (landed), with `later` taking the fragments of half h + 1.
+  // Between the StartLoad of a set of fragments and its wait there is straight-line code
+  // only - no branch, no loop edge - so the compiler has no reason to copy registers the
+  // loads have not written yet: the stores of a finished tile and the bookkeeping of the
+  // two streams, which branch, come first.
+  bool tile_complete = false;  // the half before was the last of its tile
+  auto run_half = [&](uint32_t h, const Fragments& now, Fragments& later)
+                      __attribute__((always_inline)) {
+    TileBarrier();
+    if (tile_complete) {
+      finish_tile();
+      tile_complete = false;
+    }
+    if (++half_within == 2 * nb) {
+      half_within = 0;
+      tile_complete = true;
+    }
+    const uint8_t* fragments_at = plan_next_load();
+    const CopyPlan copies = plan_next_copy();
+    __builtin_amdgcn_sched_barrier(0);
+    multiply_half(h, now, later, fragments_at, copies);
+    WaitForFragments(later);
+  };
+
   // ---- prologue: the operations the steady state would have issued before half 0 ----
   aim_copies(tile.token_tile);
   aim_loads(tile.row_tile);
-  PackedRow cur, next;
-  copy_next_half();                                   // half 0
-  if (total_halves > 1) copy_next_half();             // half 1
-  load_next_block(cur);                               // block 0
-  if (total_halves > 2) copy_next_half();             // half 2
-  WaitForRow<0>(cur);
-  next = cur;  // defined contents for the dequantization past the last block
-  SubBlockAffine(cur.header, 0, &scale, &offset);
-  bf = WeightFragment(cur, 0, scale, offset);
-
-  constexpr std::integral_constant<int, 0> kDrain{};  // unused by first halves
-  uint32_t block = 0;
-  // Steady state: every copy and load below exists, so the counts hold.
-  // Halves left whose copies were issued before the stores of a finished tile: for
-  // those the stores are kTileStores more younger operations.
-  uint32_t behind_stores = 0;
-  for (; block + 2 < total_blocks; ++block) {
-    if (behind_stores > 0) {
-      WaitVectorMemory<kEvenYounger + kTileStores>();
-      --behind_stores;
-    } else {
-      WaitVectorMemory<kEvenYounger>();
-    }
-    TileBarrier();
-    copy_next_half();
-    __builtin_amdgcn_sched_barrier(0);  // the waits count on this issue order
-    load_next_block(next);
-    multiply_half(2 * block, cur, next, std::integral_constant<int, 0>{}, kDrain);
-    if (behind_stores > 0) {
-      WaitVectorMemory<kOddYounger + kTileStores>();
-      --behind_stores;
-    } else {
-      WaitVectorMemory<kOddYounger>();
-    }
-    TileBarrier();
-    copy_next_half();
-    // Since the row loads at the top of the block: this half's copies.
-    multiply_half(2 * block + 1, cur, next, std::integral_constant<int, 1>{},
-                  std::integral_constant<int, kCopiesPerWave>{});
-    if (++block_within == nb) {
-      block_within = 0;
-      behind_stores = finish_tile() ? kAhead : 0;
-    }
-    cur = next;
+  Fragments even, odd;
+  start_copies(plan_next_copy());       // half 0
+  start_copies(plan_next_copy());       // half 1 (a tile has at least two halves)
+  {
+    const uint8_t* fragments_at = plan_next_load();  // half 0
+    const CopyPlan copies = plan_next_copy();        // half 2
+    even.StartLoad(fragments_at);
+    start_copies(copies);
   }
-  // The last two blocks: whatever copies and loads remain, complete drains.
-  for (; block < total_blocks; ++block) {
-    WaitVectorMemory<0>();
-    TileBarrier();
-    if (copy_half < total_halves) copy_next_half();
-    if (block + 1 < total_blocks) load_next_block(next);
-    multiply_half(2 * block, cur, next, std::integral_constant<int, 0>{}, kDrain);
-    WaitVectorMemory<0>();
-    TileBarrier();
-    if (copy_half < total_halves) copy_next_half();
-    multiply_half(2 * block + 1, cur, next, std::integral_constant<int, 1>{}, kDrain);
-    if (++block_within == nb) {
-      block_within = 0;
-      finish_tile();
-    }
-    cur = next;
+  WaitForFragments(even);
+  for (uint32_t h = 0; h < total_halves; h += 2) {
+    run_half(h, even, odd);
+    run_half(h + 1, odd, even);
   }
+  finish_tile();
 }
 
 }  // namespace
 
-size_t GemmWorkspaceBytes(size_t tokens, uint32_t blocks_per_row) {
-  return tokens * blocks_per_row * 256 * sizeof(_Float16);
+// Activations as fp16, then the fragments of every 32 rows of every row tile.
+size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row) {
+  const size_t act_bytes = (tokens * blocks_per_row * 512 + 255) & ~static_cast<size_t>(255);
+  const size_t row_tiles = (static_cast<size_t>(rows) + kTileRows - 1) / kTileRows;
+  return act_bytes + row_tiles * kGemmWaves * blocks_per_row * 2 * kHalfBytes;
 }
 
 hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
@@ -543,9 +593,18 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
     return hipErrorInvalidValue;
   }
   const size_t octets = tokens * blocks_per_row * 32;
-  hipLaunchKernelGGL(PrepareActivations, dim3(static_cast<uint32_t>((octets + 255) / 256)),
-                     dim3(256), 0, stream, reinterpret_cast<const U32x4*>(a_bf16), octets,
-                     static_cast<U32x4*>(workspace));
+  const size_t act_bytes = (octets * 16 + 255) & ~static_cast<size_t>(255);
+  uint8_t* a16 = static_cast<uint8_t*>(workspace);
+  uint8_t* w16 = a16 + act_bytes;
+  const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
+  const uint32_t row_groups = row_tiles * kGemmWaves;
+  const uint32_t act_groups = static_cast<uint32_t>((octets + 255) / 256);
+  // One workgroup (4 waves) per (32 rows, super-block): a wave per quarter.
+  const uint32_t weight_groups = row_groups * blocks_per_row;
+  hipLaunchKernelGGL(PrepareOperands, dim3(weight_groups + act_groups), dim3(256), 0, stream,
+                     reinterpret_cast<const U32x4*>(a_bf16), octets,
+                     reinterpret_cast<U32x4*>(a16), weight_groups, w, rows, blocks_per_row,
+                     row_groups, reinterpret_cast<U32x4*>(w16));
   hipError_t status = hipGetLastError();
   if (status != hipSuccess) return status;
 
@@ -562,7 +621,7 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
   shape.rows = rows;
   shape.nb = blocks_per_row;
   shape.tokens = static_cast<uint32_t>(tokens);
-  shape.row_tiles = (rows + kTileRows - 1) / kTileRows;
+  shape.row_tiles = row_tiles;
   shape.token_tiles = static_cast<uint32_t>((tokens + kTileTokens - 1) / kTileTokens);
   shape.band = (shape.row_tiles + kXcds - 1) / kXcds;
   shape.total = shape.row_tiles * shape.token_tiles;
@@ -573,7 +632,7 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
   if (per_xcd_groups == 0) per_xcd_groups = 1;
   if (per_xcd_groups > shape.per_xcd) per_xcd_groups = shape.per_xcd;
   hipLaunchKernelGGL(KquantGemmKernel, dim3(per_xcd_groups * kXcds), dim3(kGemmThreads),
-                     lds_bytes, stream, w, static_cast<const uint8_t*>(workspace), c, shape);
+                     lds_bytes, stream, w16, a16, c, shape);
   return hipGetLastError();
 }
 
