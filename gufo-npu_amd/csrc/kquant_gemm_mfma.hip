@@ -25,14 +25,17 @@
 //     instructions themselves: 124-133 us.  Written once as fp16 (25 MB for 6144 x 2048,
 //     5 us) the product kernel has no arithmetic left but the matrix instructions.
 //
-// Decomposition: one persistent workgroup of 8 waves per CU walks its share of the
-// 128-token x 256-row tiles.  Each wave owns 32 weight rows and multiplies them with the
-// four 32-token tiles.  The activations of half a super-block (128 tokens x 128 fp16 =
-// 32 KB, a "stage") go from global memory straight into LDS (global_load_lds_dwordx4)
-// into a ring of four stages, three halves ahead of the matrix cores - across tile
-// boundaries too, so the copies of a tile's first halves and the stores of the previous
-// tile's results overlap.  The weight operand of a half (8 steps x 16 bytes per lane)
-// comes from the pre-pass's array straight into registers, one half ahead.
+// Decomposition: one persistent workgroup of 4 waves per CU - one wave per SIMD - walks
+// its share of the 128-token x 256-row tiles.  Each wave owns 64 weight rows (two groups
+// of 32) and multiplies them with the four 32-token tiles: 8 matrix instructions per
+// step of 16 k for 4 LDS reads and 2 global loads.  (Eight waves of 32 rows each, two per
+// SIMD, read every activation fragment from LDS twice as often: 109 us against 101.)
+// The activations of half a super-block (128 tokens x 128 fp16 = 32 KB, a "stage") go
+// from global memory straight into LDS (global_load_lds_dwordx4) into a ring of four
+// stages, three halves ahead of the matrix cores - across tile boundaries too, so the
+// copies of a tile's first halves and the stores of the previous tile's results overlap.
+// The weight operand of a half (2 groups x 8 steps x 16 bytes per lane) comes from the
+// pre-pass's array straight into registers, one half ahead.
 //
 // The matrix instruction does not care which k a lane's 8 values belong to as long as
 // both operands agree, so k is dealt to lanes the way the packed block likes it: of
@@ -59,10 +62,12 @@ typedef _Float16 Half2 __attribute__((ext_vector_type(2)));
 typedef float Float16v __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* LdsPointer;
 
-constexpr int kGemmThreads = 512;
+constexpr int kGemmThreads = 256;
 constexpr int kGemmWaves = kGemmThreads / 64;
+constexpr int kWaveGroups = 2;                            // groups of 32 weight rows per wave
+constexpr int kTileGroups = kWaveGroups * kGemmWaves;     // groups of 32 weight rows per tile
 constexpr int kTileTokens = 128;
-constexpr int kTileRows = 32 * kGemmWaves;
+constexpr int kTileRows = 32 * kTileGroups;
 constexpr int kRowBytes = 256;                            // one token's half super-block as fp16
 constexpr int kStageBytes = kTileTokens * kRowBytes;      // 32 KB
 constexpr int kStages = 4;                                // the copies run kStages - 1 halves ahead
@@ -189,38 +194,40 @@ __device__ __forceinline__ uint32_t Swizzle(uint32_t t) {
 // operation - the copies into LDS that are meant to stay in flight included - once the
 // stores of a finished tile are pending in the same loop.
 struct Fragments {
-  U32x4 step[kStepsPerHalf];
+  U32x4 step[kWaveGroups][kStepsPerHalf];
 
-  // `at` is this lane's 16 bytes of step 0; the steps are kStepBytes apart.  The fields
-  // hold nothing until WaitForFragments has returned.
-  // The loads of steps 2 kPair and 2 kPair + 1 alone: the product kernel deals the eight
-  // loads of a half over the first four steps of the half before.
-  template <int kPair>
-  __device__ __forceinline__ void StartLoadPair(const uint8_t* at) {
-    static_assert(kPair >= 0 && kPair < 4, "four pairs of steps");
-    const uint8_t* base = at + (kPair / 2) * 4 * kStepBytes;
-    if constexpr (kPair % 2 == 0) {
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[2 * kPair]) : "v"(base) : "memory");
-      asm volatile("global_load_dwordx4 %0, %1, off offset:1024"
-                   : "=v"(step[2 * kPair + 1]) : "v"(base) : "memory");
+  // `at[g]` is this lane's 16 bytes of step 0 of the wave's row group g; the steps are
+  // kStepBytes apart.  The fields hold nothing until WaitForFragments has returned.
+  // The load of step kStep of row group kGroup alone: the product kernel deals the sixteen
+  // loads of a half one by one between the matrix instructions of the half before.
+  template <int kGroup, int kStep>
+  __device__ __forceinline__ void StartLoadOne(const uint8_t* const (&at)[kWaveGroups]) {
+    static_assert(kGroup >= 0 && kGroup < kWaveGroups && kStep >= 0 && kStep < kStepsPerHalf, "");
+    const uint8_t* base = at[kGroup] + (kStep / 4) * 4 * kStepBytes;  // the offset field reaches 4 KB
+    U32x4& to = step[kGroup][kStep];
+    if constexpr (kStep % 4 == 0) {
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(to) : "v"(base) : "memory");
+    } else if constexpr (kStep % 4 == 1) {
+      asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=v"(to) : "v"(base) : "memory");
+    } else if constexpr (kStep % 4 == 2) {
+      asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=v"(to) : "v"(base) : "memory");
     } else {
-      asm volatile("global_load_dwordx4 %0, %1, off offset:2048"
-                   : "=v"(step[2 * kPair]) : "v"(base) : "memory");
-      asm volatile("global_load_dwordx4 %0, %1, off offset:3072"
-                   : "=v"(step[2 * kPair + 1]) : "v"(base) : "memory");
+      asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=v"(to) : "v"(base) : "memory");
     }
   }
 
-  __device__ __forceinline__ void StartLoad(const uint8_t* at) {
-    const uint8_t* upper = at + 4 * kStepBytes;  // the offset field reaches 4 KB
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[0]) : "v"(at) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=v"(step[1]) : "v"(at) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=v"(step[2]) : "v"(at) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=v"(step[3]) : "v"(at) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(step[4]) : "v"(upper) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=v"(step[5]) : "v"(upper) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=v"(step[6]) : "v"(upper) : "memory");
-    asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=v"(step[7]) : "v"(upper) : "memory");
+  // Load number kIndex (0..15) of a half, in the order the product kernel issues them.
+  template <int kIndex>
+  __device__ __forceinline__ void StartLoadNumber(const uint8_t* const (&at)[kWaveGroups]) {
+    StartLoadOne<kIndex % kWaveGroups, kIndex / kWaveGroups>(at);
+  }
+
+  template <int kIndex = 0>
+  __device__ __forceinline__ void StartLoad(const uint8_t* const (&at)[kWaveGroups]) {
+    if constexpr (kIndex < kWaveGroups * kStepsPerHalf) {
+      StartLoadNumber<kIndex>(at);
+      StartLoad<kIndex + 1>(at);
+    }
   }
 };
 static_assert(kStepBytes == 1024 && kStepsPerHalf == 8, "the offsets above");
@@ -230,10 +237,17 @@ static_assert(kStepBytes == 1024 && kStepsPerHalf == 8, "the offsets above");
 // copies and stores alike, so everything older has landed too).  Ties the fields to the
 // wait so that no use of them moves above it.
 __device__ __forceinline__ void WaitForFragments(Fragments& f) {
-  static_assert(kCopiesPerWave == 4, "update the literal below");
-  asm volatile("s_waitcnt vmcnt(4)"
-               : "+v"(f.step[0]), "+v"(f.step[1]), "+v"(f.step[2]), "+v"(f.step[3]),
-                 "+v"(f.step[4]), "+v"(f.step[5]), "+v"(f.step[6]), "+v"(f.step[7])
+  static_assert(kCopiesPerWave == 8 && kWaveGroups == 2, "update the literal and the lists below");
+  asm volatile("s_waitcnt vmcnt(8)"
+               : "+v"(f.step[0][0]), "+v"(f.step[0][1]), "+v"(f.step[0][2]), "+v"(f.step[0][3]),
+                 "+v"(f.step[0][4]), "+v"(f.step[0][5]), "+v"(f.step[0][6]), "+v"(f.step[0][7])
+               :
+               : "memory");
+  // (An asm statement takes 30 operands at most; the second group is tied to the point
+  // behind the wait by a statement of its own.)
+  asm volatile(""
+               : "+v"(f.step[1][0]), "+v"(f.step[1][1]), "+v"(f.step[1][2]), "+v"(f.step[1][3]),
+                 "+v"(f.step[1][4]), "+v"(f.step[1][5]), "+v"(f.step[1][6]), "+v"(f.step[1][7])
                :
                : "memory");
 }
@@ -249,31 +263,35 @@ __device__ __forceinline__ uint32_t LdsAddress(const uint8_t* p) {
 struct ActivationFragments {
   U32x4 tile[4];
 
-  __device__ __forceinline__ void StartRead(uint32_t at) {
+  template <int kTile>
+  __device__ __forceinline__ void StartReadOne(uint32_t at) {
     static_assert(32 * kRowBytes == 8192, "the offsets below");
-    asm volatile("ds_read_b128 %0, %1" : "=v"(tile[0]) : "v"(at) : "memory");
-    asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(tile[1]) : "v"(at) : "memory");
-    asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(tile[2]) : "v"(at) : "memory");
-    asm volatile("ds_read_b128 %0, %1 offset:24576" : "=v"(tile[3]) : "v"(at) : "memory");
+    if constexpr (kTile == 0) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(tile[0]) : "v"(at) : "memory");
+    } else if constexpr (kTile == 1) {
+      asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(tile[1]) : "v"(at) : "memory");
+    } else if constexpr (kTile == 2) {
+      asm volatile("ds_read_b128 %0, %1 offset:16384" : "=v"(tile[2]) : "v"(at) : "memory");
+    } else {
+      static_assert(kTile == 3, "four tiles");
+      asm volatile("ds_read_b128 %0, %1 offset:24576" : "=v"(tile[3]) : "v"(at) : "memory");
+    }
+  }
+
+  __device__ __forceinline__ void StartRead(uint32_t at) {
+    StartReadOne<0>(at);
+    StartReadOne<1>(at);
+    StartReadOne<2>(at);
+    StartReadOne<3>(at);
   }
 };
 
-// Waits until at most kYounger LDS reads issued after f's are outstanding (LDS reads
-// return in order): 4 when the next step's reads follow, 0 for the last step of a half.
-template <int kYounger>
+// Waits until every LDS read issued so far has returned.
 __device__ __forceinline__ void WaitForActivations(ActivationFragments& f) {
-  static_assert(kYounger == 0 || kYounger == 4, "the counts the step loop produces");
-  if constexpr (kYounger == 0) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(f.tile[0]), "+v"(f.tile[1]), "+v"(f.tile[2]), "+v"(f.tile[3])
-                 :
-                 : "memory");
-  } else {
-    asm volatile("s_waitcnt lgkmcnt(4)"
-                 : "+v"(f.tile[0]), "+v"(f.tile[1]), "+v"(f.tile[2]), "+v"(f.tile[3])
-                 :
-                 : "memory");
-  }
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(f.tile[0]), "+v"(f.tile[1]), "+v"(f.tile[2]), "+v"(f.tile[3])
+               :
+               : "memory");
 }
 
 // The 16-byte piece of a token's half super-block that step s (0..7 within the half)
@@ -291,7 +309,6 @@ struct GemmShape {
   uint32_t band;         // weight-row tiles per band; the last band may hold fewer
   uint32_t per_xcd;      // consecutive tiles of the order each XCD takes
   uint32_t total;        // row_tiles * token_tiles
-  uint32_t vector_stores;  // c and its rows are 16-byte aligned
 };
 
 struct TileCoord {
@@ -326,18 +343,20 @@ __device__ __forceinline__ void TileBarrier() {
   asm volatile("" ::: "memory");
 }
 
-// One workgroup per CU (the stage ring takes 128 KB of LDS): 2 waves per SIMD.
+// One workgroup per CU (the stage ring takes 128 KB of LDS): one wave per SIMD, which
+// leaves it the whole register file - 128 accumulator registers, two sets of 64 for the
+// weight fragments.
 //
 // The stream: this workgroup's tiles one after the other, each 2 nb halves.  Per wave,
 // every half issues the same vector-memory operations in the same order - after the
 // barrier the stores of the tile the half before completed (if any), then the weight
-// fragments of half h + 1 (8 loads), then the copies of half h + 3 (kCopiesPerWave
+// fragments of half h + 1 (16 loads), then the copies of half h + 3 (kCopiesPerWave
 // instructions) - and, after its matrix instructions, waits until only those copies may
 // still be in flight: the fragments of half h + 1 have then landed, and with them
 // everything older, the copies of half h + 1 among it.  Past the end of the stream the
 // loads and copies repeat the last half into registers and a stage nobody uses, so the
 // count never changes.
-__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void
 KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a16,
                  float* __restrict__ c, GemmShape shape) {
   extern __shared__ __align__(1024) uint8_t stages[];  // kStages x kStageBytes
@@ -408,17 +427,25 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
 
   // ---- weight fragments, one half ahead ----
   // Past the end of the stream the last half is loaded again and never used.
-  const uint8_t* load_ptr = nullptr;  // this lane's 16 bytes of step 0 of the next half to load
+  // This lane's 16 bytes of step 0 of the next half to load, in the wave's first row
+  // group; the fragments of its other groups follow group_bytes apart.
+  const uint8_t* load_ptr = nullptr;
+  const size_t group_bytes = static_cast<size_t>(nb) * 2 * kHalfBytes;
   uint32_t load_half = 0;
   uint32_t load_within = 0;
   uint32_t load_tile = 0;
   auto aim_loads = [&](uint32_t row_tile) __attribute__((always_inline)) {
-    const size_t group = static_cast<size_t>(row_tile) * kGemmWaves + wave;
-    load_ptr = w16 + group * nb * 2 * kHalfBytes + lane * 16;
+    const size_t group = static_cast<size_t>(row_tile) * kTileGroups + wave * kWaveGroups;
+    load_ptr = w16 + group * group_bytes + lane * 16;
+  };
+  struct LoadPlan {
+    const uint8_t* at[kWaveGroups];
   };
   // Where the fragments of the next half are; moves on to the half after it.
   auto plan_next_load = [&]() __attribute__((always_inline)) {
-    const uint8_t* at = load_ptr;
+    LoadPlan plan;
+#pragma unroll
+    for (int g = 0; g < kWaveGroups; ++g) plan.at[g] = load_ptr + g * group_bytes;
     if (++load_half < total_halves) {
       load_ptr += kHalfBytes;
       if (++load_within == 2 * nb) {
@@ -427,15 +454,18 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
         aim_loads(DecodeTile(shape, first + load_tile * stride).row_tile);
       }
     }
-    return at;
+    return plan;
   };
 
-  Float16v acc[4];
+  Float16v acc[kWaveGroups][4];
   auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
+    for (int g = 0; g < kWaveGroups; ++g) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+      for (int m = 0; m < 4; ++m) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[g][m][i] = 0.0f;
+      }
     }
   };
   clear_acc();
@@ -445,46 +475,80 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
   const uint32_t flip = Swizzle(n & 15u) ^ (u << 1);
   const uint32_t read_base = n * kRowBytes;
 
-  // One half super-block: 8 steps on the stage of stream half `half`.  While step s
-  // multiplies, the activation fragments of step s + 1 are on their way from LDS: the
-  // reads of step s + 1 are issued, then the wait lets exactly those four stay in flight.
-  // (Left to the compiler the wait becomes lgkmcnt(0) on every second step, which puts a
-  // whole LDS latency in front of the matrix instructions: 55% of the waves' time.)
-  //
-  // The half's vector-memory operations ride along, behind the matrix instructions of
-  // the steps: the next half's weight fragments two loads a step over steps 0-3, the
-  // copies of the half three ahead one a step over steps 4-7.  Issued in one burst after
-  // the barrier - when all eight waves of the workgroup are at the same point - they
-  // queued up at the one address unit with no matrix instruction to cover them (measured:
-  // 46 of 115 us).
+  // The constant-index members behind indices that are constants only once the step loop
+  // is unrolled.
+  auto start_read_one = [&](ActivationFragments& f, int m, uint32_t at)
+                            __attribute__((always_inline)) {
+    switch (m) {
+      case 0: f.template StartReadOne<0>(at); break;
+      case 1: f.template StartReadOne<1>(at); break;
+      case 2: f.template StartReadOne<2>(at); break;
+      default: f.template StartReadOne<3>(at); break;
+    }
+  };
+  auto start_load_number = [&](Fragments& f, const LoadPlan& at, int index)
+                               __attribute__((always_inline)) {
+    switch (index) {
+      case 0: f.template StartLoadNumber<0>(at.at); break;
+      case 1: f.template StartLoadNumber<1>(at.at); break;
+      case 2: f.template StartLoadNumber<2>(at.at); break;
+      case 3: f.template StartLoadNumber<3>(at.at); break;
+      case 4: f.template StartLoadNumber<4>(at.at); break;
+      case 5: f.template StartLoadNumber<5>(at.at); break;
+      case 6: f.template StartLoadNumber<6>(at.at); break;
+      case 7: f.template StartLoadNumber<7>(at.at); break;
+      case 8: f.template StartLoadNumber<8>(at.at); break;
+      case 9: f.template StartLoadNumber<9>(at.at); break;
+      case 10: f.template StartLoadNumber<10>(at.at); break;
+      case 11: f.template StartLoadNumber<11>(at.at); break;
+      case 12: f.template StartLoadNumber<12>(at.at); break;
+      case 13: f.template StartLoadNumber<13>(at.at); break;
+      case 14: f.template StartLoadNumber<14>(at.at); break;
+      default: f.template StartLoadNumber<15>(at.at); break;
+    }
+  };
+
+  // One half super-block: 8 steps of 8 matrix instructions on the stage of stream half
+  // `half`.  A wave is alone on its SIMD, so whatever it issues between two matrix
+  // instructions is covered by the first of them (32 cycles in the matrix core), and
+  // whatever it issues in a block of its own is not.  Hence one memory instruction behind
+  // each matrix instruction: behind the first four of step s the LDS reads of step s + 1's
+  // activation fragments, behind the last four a quarter of the half's vector-memory
+  // operations - the next half's weight fragments over steps 0-3, the copies of the half
+  // three ahead over steps 4-7 (two a step).  The wait at the top of a step is then for
+  // reads that were issued at least four matrix instructions earlier.
+  // (Left to the compiler, the LDS waits become lgkmcnt(0) right behind the reads on every
+  // second step: a whole LDS latency in front of the matrix instructions.)
   auto multiply_half = [&](uint32_t half, const Fragments& weights, Fragments& later,
-                           const uint8_t* later_at, const CopyPlan& copies)
+                           const LoadPlan& later_at, const CopyPlan& copies)
                            __attribute__((always_inline)) {
     const uint32_t tile = LdsAddress(stages + (half % kStages) * kStageBytes + read_base);
     ActivationFragments af[2];
     af[0].StartRead(tile + ((StepPiece(0) ^ flip) << 4));
 #pragma unroll
     for (int s = 0; s < kStepsPerHalf; ++s) {
-      if (s + 1 < kStepsPerHalf) {
-        af[(s + 1) & 1].StartRead(tile + ((StepPiece(s + 1) ^ flip) << 4));
-        WaitForActivations<4>(af[s & 1]);
-      } else {
-        WaitForActivations<0>(af[s & 1]);
-      }
-      const Half8 bf = __builtin_bit_cast(Half8, weights.step[s]);
+      WaitForActivations(af[s & 1]);
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-            bf, __builtin_bit_cast(Half8, af[s & 1].tile[m]), acc[m], 0, 0, 0);
+      for (int j = 0; j < 4 * kWaveGroups; ++j) {
+        const int g = j % kWaveGroups;
+        const int m = j / kWaveGroups;
+        acc[g][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            __builtin_bit_cast(Half8, af[s & 1].tile[m]),
+            __builtin_bit_cast(Half8, weights.step[g][s]), acc[g][m], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j < 4) {
+          // Into the registers step s - 1 multiplied from: its last matrix instruction was
+          // issued before this step's first.
+          if (s + 1 < kStepsPerHalf) {
+            start_read_one(af[(s + 1) & 1], j, tile + ((StepPiece(s + 1) ^ flip) << 4));
+          }
+        } else if (s < 4) {
+          start_load_number(later, later_at, 4 * s + (j - 4));
+        } else if (j - 4 < 2) {
+          start_copy(copies, 2 * (s - 4) + (j - 4));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // the wait of the half counts on this issue order
       }
-      // The reads of step s + 2 reuse this step's registers: not before it has multiplied.
-      __builtin_amdgcn_sched_barrier(0);
-      if (s == 0) later.template StartLoadPair<0>(later_at);
-      if (s == 1) later.template StartLoadPair<1>(later_at);
-      if (s == 2) later.template StartLoadPair<2>(later_at);
-      if (s == 3) later.template StartLoadPair<3>(later_at);
-      if (s >= 4) start_copy(copies, s - 4);
-      __builtin_amdgcn_sched_barrier(0);  // the wait of the half counts on this issue order
     }
   };
 
@@ -492,43 +556,41 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
   uint32_t tile_index = 0;
   uint32_t half_within = 0;
   TileCoord tile = DecodeTile(shape, first);
-  // With the weights as the first operand, accumulator register i of token tile m holds
-  // weight row 8 (i/4) + 4 u + i%4 of this wave's 32 and token 32 m + n: four registers
-  // are four consecutive floats of a row of c.  A tile that lies wholly inside c stores
-  // them as kTileStores 16-byte stores per wave; a ragged one stores float by float.
-  // Returns whether the fixed number of stores was issued.
-  auto finish_tile = [&]() __attribute__((always_inline)) -> bool {
-    const uint32_t row0 = tile.row_tile * kTileRows + wave * 32;
+  // With the activations as the first operand, accumulator register i of row group g,
+  // token tile m holds token 32 m + 8 (i/4) + 4 u + i%4 and weight row 32 g + n of this
+  // wave's 64: a store instruction writes, for two tokens (u = 0, 1), 32 consecutive
+  // floats of their rows of c each - whole 128-byte lines when the matrix has a multiple
+  // of 32 rows.
+  auto finish_tile = [&]() __attribute__((always_inline)) {
+    const uint32_t row0 = tile.row_tile * kTileRows + wave * (32 * kWaveGroups);
     const uint32_t token_first = tile.token_tile * kTileTokens;
-    const bool whole = shape.vector_stores != 0 && row0 + 32 <= shape.rows &&
+    const bool whole = row0 + 32 * kWaveGroups <= shape.rows &&
                        token_first + kTileTokens <= shape.tokens;
-    if (whole) {
+    auto store_all = [&](auto check) __attribute__((always_inline)) {
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        float* at = c + static_cast<size_t>(token_first + m * 32 + n) * shape.rows + row0 + 4 * u;
+      for (int g = 0; g < kWaveGroups; ++g) {
+        const uint32_t row = row0 + 32 * g + n;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          typedef float Float4 __attribute__((ext_vector_type(4)));
-          const Float4 v = {acc[m][4 * q], acc[m][4 * q + 1], acc[m][4 * q + 2], acc[m][4 * q + 3]};
-          *reinterpret_cast<Float4*>(at + 8 * q) = v;
-        }
-      }
-    } else {
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t t0 = token_first + m * 32 + 4 * u;
+          float* at = c + static_cast<size_t>(t0) * shape.rows + row;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const uint32_t t = token_first + m * 32 + n;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const uint32_t row = row0 + 8 * (i >> 2) + 4 * u + (i & 3);
-          if (t < shape.tokens && row < shape.rows) {
-            c[static_cast<size_t>(t) * shape.rows + row] = acc[m][i];
+          for (int i = 0; i < 16; ++i) {
+            const uint32_t dt = 8 * (i >> 2) + (i & 3);
+            if (!decltype(check)::value || (t0 + dt < shape.tokens && row < shape.rows)) {
+              at[static_cast<size_t>(dt) * shape.rows] = acc[g][m][i];
+            }
           }
         }
       }
+    };
+    if (whole) {
+      store_all(std::false_type{});
+    } else {
+      store_all(std::true_type{});
     }
     clear_acc();
     if (++tile_index < n_tiles) tile = DecodeTile(shape, first + tile_index * stride);
-    return whole;
   };
 
   // Stream half h on `now` (landed), with `later` taking the fragments of half h + 1.
@@ -548,7 +610,7 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
       half_within = 0;
       tile_complete = true;
     }
-    const uint8_t* fragments_at = plan_next_load();
+    const LoadPlan fragments_at = plan_next_load();
     const CopyPlan copies = plan_next_copy();
     __builtin_amdgcn_sched_barrier(0);
     multiply_half(h, now, later, fragments_at, copies);
@@ -562,9 +624,9 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
   start_copies(plan_next_copy());       // half 0
   start_copies(plan_next_copy());       // half 1 (a tile has at least two halves)
   {
-    const uint8_t* fragments_at = plan_next_load();  // half 0
+    const LoadPlan fragments_at = plan_next_load();  // half 0
     const CopyPlan copies = plan_next_copy();        // half 2
-    even.StartLoad(fragments_at);
+    even.StartLoad(fragments_at.at);
     start_copies(copies);
   }
   WaitForFragments(even);
@@ -581,7 +643,7 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
 size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row) {
   const size_t act_bytes = (tokens * blocks_per_row * 512 + 255) & ~static_cast<size_t>(255);
   const size_t row_tiles = (static_cast<size_t>(rows) + kTileRows - 1) / kTileRows;
-  return act_bytes + row_tiles * kGemmWaves * blocks_per_row * 2 * kHalfBytes;
+  return act_bytes + row_tiles * kTileGroups * blocks_per_row * 2 * kHalfBytes;
 }
 
 hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
@@ -597,7 +659,7 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
   uint8_t* a16 = static_cast<uint8_t*>(workspace);
   uint8_t* w16 = a16 + act_bytes;
   const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
-  const uint32_t row_groups = row_tiles * kGemmWaves;
+  const uint32_t row_groups = row_tiles * kTileGroups;
   const uint32_t act_groups = static_cast<uint32_t>((octets + 255) / 256);
   // One workgroup (4 waves) per (32 rows, super-block): a wave per quarter.
   const uint32_t weight_groups = row_groups * blocks_per_row;
@@ -626,7 +688,6 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
   shape.band = (shape.row_tiles + kXcds - 1) / kXcds;
   shape.total = shape.row_tiles * shape.token_tiles;
   shape.per_xcd = (shape.total + kXcds - 1) / kXcds;
-  shape.vector_stores = (rows % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0) ? 1 : 0;
   // One workgroup per CU, the same number on every XCD, no more than there are tiles.
   uint32_t per_xcd_groups = static_cast<uint32_t>(DeviceComputeUnits()) / kXcds;
   if (per_xcd_groups == 0) per_xcd_groups = 1;
