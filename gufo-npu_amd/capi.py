@@ -100,6 +100,8 @@ SIGNATURES = {
     "gufo_hip_moe_ffn": (C.c_int, [_P, _P, _P, C.c_int, _P, C.c_int, _P, _P, C.c_int, _P]),
     "gufo_hip_moe_ffn_dev": (C.c_int, [_P, _P, _P, C.c_int, _P, C.c_int, _P, _P, C.c_int,
                                        _P]),
+    "gufo_hip_gemm_bf16": (C.c_int, [_P, _P, _SZ, _P]),
+    "gufo_hip_gemm_bf16_dev": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_q4k_bf16": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_q4k_bf16_dev": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_capture_begin": (C.c_int, []),
@@ -387,6 +389,20 @@ def route_topk_dev(logits: DeviceBuffer, tokens: int, experts: int, k: int,
                    ids: DeviceBuffer, weights: DeviceBuffer) -> None:
     _check(load_library().gufo_hip_route_topk_dev(C.c_void_p(logits.ptr), tokens, experts, k,
                                                   C.c_void_p(ids.ptr), C.c_void_p(weights.ptr)))
+
+
+def gemm_bf16(w: Matrix, a_bf16: np.ndarray) -> np.ndarray:
+    """The prefill product for rows of any quantized type (gufo_hip_gemm_bf16)."""
+    a_bf16 = np.ascontiguousarray(a_bf16, dtype=np.uint16)
+    m = a_bf16.shape[0]
+    c = np.empty((m, w.rows), dtype=np.float32)
+    _check(load_library().gufo_hip_gemm_bf16(C.c_void_p(w.handle), _ptr(a_bf16), m, _ptr(c)))
+    return c
+
+
+def gemm_bf16_dev(w: Matrix, a: DeviceBuffer, m: int, c: DeviceBuffer) -> None:
+    _check(load_library().gufo_hip_gemm_bf16_dev(C.c_void_p(w.handle), C.c_void_p(a.ptr), m,
+                                                 C.c_void_p(c.ptr)))
 
 
 def gemm_q4k_bf16(w: Matrix, a_bf16: np.ndarray) -> np.ndarray:

@@ -1021,11 +1021,18 @@ int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
 
 namespace {
 
-int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* c) {
+int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* c,
+                  bool q4k_only) {
   if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
-  if (w->type != GUFO_HIP_Q4_K) {
+  if (q4k_only && w->type != GUFO_HIP_Q4_K) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
-                "the prefill GEMM takes Q4_K weights; this matrix has ggml type %d", w->type);
+                "this entry point takes Q4_K weights; this matrix has ggml type %d", w->type);
+  }
+  if (!gufo::GemmTakesType(w->type)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "the prefill GEMM takes Q4_K, Q5_K, Q6_K or Q8_0 weights; this matrix has "
+                "ggml type %d",
+                w->type);
   }
   if (m == 0 || w->rows == 0) return GUFO_HIP_OK;
   if (a == nullptr || c == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a or c is null");
@@ -1035,24 +1042,13 @@ int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* 
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens exceed the launch limit", m);
   }
   GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmWorkspaceBytes(m, static_cast<uint32_t>(w->rows), nb)));
-  GUFO_HIP_TRY(gufo::LaunchGemmQ4K(w->data, static_cast<uint32_t>(w->rows), nb, a, m,
-                                   g_state.gemm_work.ptr, c, g_state.stream));
+  GUFO_HIP_TRY(gufo::LaunchGemm(w->type, w->data, static_cast<uint32_t>(w->rows), nb, a, m,
+                                g_state.gemm_work.ptr, c, g_state.stream));
   return GUFO_HIP_OK;
 }
 
-}  // namespace
-
-int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
-                               size_t m, float* c_dev) {
-  const std::lock_guard<std::mutex> lock(g_state.mutex);
-  GUFO_TRY(RequireReady());
-  return GemmDevLocked(w, a_bf16_dev, m, c_dev);
-}
-
-int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
-                           float* c_host) {
-  const std::lock_guard<std::mutex> lock(g_state.mutex);
-  GUFO_TRY(RequireReady());
+int GemmHostLocked(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
+                   float* c_host, bool q4k_only) {
   if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
   if (m == 0 || w->rows == 0) return GUFO_HIP_OK;
   if (a_bf16_host == nullptr || c_host == nullptr) {
@@ -1063,8 +1059,38 @@ int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host
   GUFO_TRY(CopyIn(&g_state.stage_x, a_bf16_host, a_bytes));
   GUFO_TRY(Reserve(&g_state.stage_c, c_bytes));
   GUFO_TRY(GemmDevLocked(w, static_cast<const uint16_t*>(g_state.stage_x.ptr), m,
-                         static_cast<float*>(g_state.stage_c.ptr)));
+                         static_cast<float*>(g_state.stage_c.ptr), q4k_only));
   return CopyOut(c_host, g_state.stage_c.ptr, c_bytes);
+}
+
+}  // namespace
+
+int gufo_hip_gemm_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev, size_t m,
+                           float* c_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemmDevLocked(w, a_bf16_dev, m, c_dev, false);
+}
+
+int gufo_hip_gemm_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
+                       float* c_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemmHostLocked(w, a_bf16_host, m, c_host, false);
+}
+
+int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
+                               size_t m, float* c_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemmDevLocked(w, a_bf16_dev, m, c_dev, true);
+}
+
+int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
+                           float* c_host) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemmHostLocked(w, a_bf16_host, m, c_host, true);
 }
 
 int gufo_hip_capture_begin(void) {

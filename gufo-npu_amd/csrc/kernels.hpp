@@ -166,14 +166,17 @@ hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const
 
 // ---- prefill ------------------------------------------------------------------
 
-// Bytes of device workspace LaunchGemmQ4K needs: both operands as fp16.
+// Bytes of device workspace LaunchGemm needs: both operands as fp16.
 size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row);
 
-// c[t*rows + r] = row r of the Q4_K matrix w . a[t], a given as bf16 (tokens x
-// blocks_per_row*256), on the matrix cores with fp32 accumulation.
-hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
-                         const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
-                         hipStream_t stream);
+// Row types LaunchGemm takes: Q4_K, Q5_K, Q6_K, Q8_0.
+bool GemmTakesType(int type);
+
+// c[t*rows + r] = row r of the matrix w (rows of `type`) . a[t], a given as bf16
+// (tokens x blocks_per_row*256), on the matrix cores with fp32 accumulation.
+hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
+                      const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
+                      hipStream_t stream);
 
 // index of the first maximum of v[0..n) -> *out (device); scratch holds
 // 2*kArgmaxBlocks entries of 8 bytes.

@@ -1,10 +1,12 @@
-// Prefill projection on the matrix cores: C[t][r] = row r of a Q4_K matrix . a[t]
+// Prefill projection on the matrix cores: C[t][r] = row r of a quantized matrix . a[t]
 // for many tokens, a given as bf16.  This is GgufProjections::MatMul with
 // tokens = m (src/models/qwen35/gguf_projections.cpp:239-286 of the reference), the
 // shape the reference's NPU serves with its prefill GEMM (src/npu/gemm.hpp:99-105).
 //
 // Two launches.  A pre-pass turns both operands into fp16 once per call; the product
-// kernel then only moves 16-bit operands and issues matrix instructions.
+// kernel then only moves 16-bit operands and issues matrix instructions, whatever the
+// row type was (Q4_K, Q5_K, Q6_K, Q8_0).  For Q4_K, the type of the prefill
+// configuration, the pre-pass is written around the packed block:
 //
 //   weight[r][k] = d * sc_j * q - dmin * m_j          (j = sub-block of k)
 //
@@ -75,7 +77,6 @@ constexpr int kCopiesPerWave = kStageBytes / 1024 / kGemmWaves;  // 1 KB per wav
 constexpr int kStepsPerHalf = 8;
 constexpr int kStepBytes = 64 * 16;                       // one step's fragments of 32 rows
 constexpr int kHalfBytes = kStepsPerHalf * kStepBytes;    // 8 KB per 32 rows and half super-block
-constexpr int kQ4Block = 144;
 constexpr int kXcds = 8;
 
 // ---- pre-pass ---------------------------------------------------------------------
@@ -124,12 +125,94 @@ __device__ __forceinline__ U32x4 WeightFragment(const U32x4& codes, int q, float
   return out;
 }
 
+// The other row types: the 8 weights k0 .. k0 + 7 (k0 a multiple of 8) of the 256 values
+// that start at `blk`, in fp32.  Eight such neighbours share a sub-block in every format,
+// and their codes are 8 consecutive bytes.  Each weight is exact in fp32 or rounded once
+// (the K-quant formulas of src/core/quant.cpp:61-133 of the reference, Q8_0 of :22-31).
+template <int TYPE>
+__device__ __forceinline__ void DequantEight(const uint8_t* blk, uint32_t k0, float (&out)[8]) {
+  if constexpr (TYPE == kTypeQ5K) {
+    // d, dmin | 12 scale bytes | qh[32] | qs[128]: value k of the 64 values 64 p .. is the
+    // low (k % 64 < 32) or high nibble of qs[32 p + k % 32] plus 16 x bit (2 p + high) of
+    // qh[k % 32].
+    const uint32_t p = k0 >> 6;
+    const uint32_t high = (k0 >> 5) & 1u;
+    const uint32_t l = k0 & 31u;
+    const U32x4 header = Load16(blk);
+    float scale, offset;
+    {
+      const float d = HalfBitsToFloat(header.x & 0xFFFFu);
+      const float dmin = HalfBitsToFloat(header.x >> 16);
+      uint32_t sc, mn;
+      ScaleMinK4(header.y, header.z, header.w, static_cast<int>(2 * p + high), &sc, &mn);
+      scale = d * static_cast<float>(sc);
+      offset = -dmin * static_cast<float>(mn);
+    }
+    const U32x2 qs = Load8Align2(blk + 48 + 32 * p + l);
+    const U32x2 qh = Load8Align2(blk + 16 + l);
+    const uint32_t codes[2] = {qs.x >> (4 * high), qs.y >> (4 * high)};
+    const uint32_t fifth[2] = {qh.x >> (2 * p + high), qh.y >> (2 * p + high)};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t q = ((codes[i >> 2] >> (8 * (i & 3))) & 15u) +
+                         (((fifth[i >> 2] >> (8 * (i & 3))) & 1u) << 4);
+      out[i] = __builtin_fmaf(static_cast<float>(q), scale, offset);
+    }
+  } else if constexpr (TYPE == kTypeQ6K) {
+    // ql[128] | qh[64] | int8 scales[16] | d: of each 128 values, quarter c (32 values)
+    // takes the low (c < 2) or high nibble of ql[64 n + 32 (c & 1) + l] and bits 2 c,
+    // 2 c + 1 of qh[32 n + l]; scale 8 n + 2 c + l / 16.
+    const uint32_t n = k0 >> 7;
+    const uint32_t c = (k0 >> 5) & 3u;
+    const uint32_t l = k0 & 31u;
+    const U32x2 ql = Load8Align2(blk + 64 * n + 32 * (c & 1u) + l);
+    const U32x2 qh = Load8Align2(blk + 128 + 32 * n + l);
+    const int sc = static_cast<int8_t>(blk[192 + 8 * n + 2 * c + (l >> 4)]);
+    const float d = HalfBitsToFloat(Load2(blk + 208));
+    const uint32_t low[2] = {ql.x >> (4 * (c >> 1)), ql.y >> (4 * (c >> 1))};
+    const uint32_t top[2] = {qh.x >> (2 * c), qh.y >> (2 * c)};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = static_cast<int>(((low[i >> 2] >> (8 * (i & 3))) & 15u) |
+                                     (((top[i >> 2] >> (8 * (i & 3))) & 3u) << 4)) - 32;
+      out[i] = d * static_cast<float>(sc * q);  // 11 x 13 bits: exact
+    }
+  } else {
+    static_assert(TYPE == kTypeQ80, "Q5_K, Q6_K or Q8_0");
+    // Eight blocks of d | 32 int8.
+    const uint8_t* sub = blk + 34 * (k0 >> 5);
+    const float d = HalfBitsToFloat(Load2(sub));
+    const U32x2 q = Load8Align2(sub + 2 + (k0 & 31u));
+    const uint32_t words[2] = {q.x, q.y};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int v = static_cast<int8_t>((words[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+      out[i] = d * static_cast<float>(v);  // 11 x 8 bits: exact
+    }
+  }
+}
+
+// Eight fp32 weights as one fragment: fp16, round to nearest, magnitudes above 65504
+// saturate.
+__device__ __forceinline__ U32x4 PackFragment(const float (&v)[8]) {
+  uint32_t packed[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = __builtin_fminf(__builtin_fmaxf(v[2 * i], -65504.0f), 65504.0f);
+    const float hi = __builtin_fminf(__builtin_fmaxf(v[2 * i + 1], -65504.0f), 65504.0f);
+    const Half2 h = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+    packed[i] = __builtin_bit_cast(uint32_t, h);
+  }
+  return U32x4{packed[0], packed[1], packed[2], packed[3]};
+}
+
 // Both operands as fp16, one launch.  Every wave of workgroups [0, weight_groups)
 // dequantizes a quarter (64 values, 4 steps) of one super-block of one group of 32 rows
 // into fragments: w16[((group * nb + block) * 16 + step) * 64 + lane] (16 bytes each);
 // rows past the matrix repeat its last row, their products are not stored.  The other
 // workgroups convert 256 octets of activations each (bf16 -> fp16, same [token][k]
 // layout).
+template <int TYPE>
 __global__ __launch_bounds__(256) void PrepareOperands(
     const U32x4* __restrict__ a, size_t octets, U32x4* __restrict__ a16,
     uint32_t weight_groups, const uint8_t* __restrict__ w, uint32_t rows, uint32_t nb,
@@ -162,17 +245,28 @@ __global__ __launch_bounds__(256) void PrepareOperands(
   const uint32_t n = lane & 31;
   const uint32_t u = lane >> 5;
   const uint32_t r = min(group * 32 + n, rows - 1);
-  const uint8_t* blk = w + (static_cast<size_t>(r) * nb + block) * kQ4Block;
-  const U32x4 header = Load16(blk);
-  const U32x4 codes = Load16(blk + 16 + 32 * p + 16 * u);
+  const uint8_t* blk = w + (static_cast<size_t>(r) * nb + block) * BlockBytes(TYPE);
   U32x4* out = w16 + (static_cast<size_t>(unit) * 16 + 4 * p) * 64 + lane;
+  if constexpr (TYPE == kTypeQ4K) {
+    const U32x4 header = Load16(blk);
+    const U32x4 codes = Load16(blk + 16 + 32 * p + 16 * u);
 #pragma unroll
-  for (int high = 0; high < 2; ++high) {
-    float scale, offset;
-    SubBlockAffine(header, 2 * p + high, &scale, &offset);
+    for (int high = 0; high < 2; ++high) {
+      float scale, offset;
+      SubBlockAffine(header, 2 * p + high, &scale, &offset);
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      out[(2 * high + half) * 64] = WeightFragment(codes, 2 * high + half, scale, offset);
+      for (int half = 0; half < 2; ++half) {
+        out[(2 * high + half) * 64] = WeightFragment(codes, 2 * high + half, scale, offset);
+      }
+    }
+  } else {
+    // Step 4 p + q holds k = 64 p + 32 (q / 2) + 16 u + 8 (q % 2) .. + 8, the order the
+    // packed Q4_K block suggested; the activation side reads its pieces to match.
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float v[8];
+      DequantEight<TYPE>(blk, 64 * p + 32 * (q >> 1) + 16 * u + 8 * (q & 1), v);
+      out[q * 64] = PackFragment(v);
     }
   }
 }
@@ -646,9 +740,14 @@ size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row)
   return act_bytes + row_tiles * kTileGroups * blocks_per_row * 2 * kHalfBytes;
 }
 
-hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
-                         const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
-                         hipStream_t stream) {
+bool GemmTakesType(int type) {
+  return type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ80;
+}
+
+hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
+                      const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
+                      hipStream_t stream) {
+  if (!GemmTakesType(type)) return hipErrorInvalidValue;
   if (rows == 0 || tokens == 0) return hipSuccess;
   // Activation bytes are addressed with 32 bits.
   if (blocks_per_row == 0 || tokens > 0xFFFFFFFFull / (512ull * blocks_per_row)) {
@@ -663,10 +762,18 @@ hipError_t LaunchGemmQ4K(const uint8_t* w, uint32_t rows, uint32_t blocks_per_ro
   const uint32_t act_groups = static_cast<uint32_t>((octets + 255) / 256);
   // One workgroup (4 waves) per (32 rows, super-block): a wave per quarter.
   const uint32_t weight_groups = row_groups * blocks_per_row;
-  hipLaunchKernelGGL(PrepareOperands, dim3(weight_groups + act_groups), dim3(256), 0, stream,
-                     reinterpret_cast<const U32x4*>(a_bf16), octets,
-                     reinterpret_cast<U32x4*>(a16), weight_groups, w, rows, blocks_per_row,
-                     row_groups, reinterpret_cast<U32x4*>(w16));
+  auto prepare = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(weight_groups + act_groups), dim3(256), 0, stream,
+                       reinterpret_cast<const U32x4*>(a_bf16), octets,
+                       reinterpret_cast<U32x4*>(a16), weight_groups, w, rows, blocks_per_row,
+                       row_groups, reinterpret_cast<U32x4*>(w16));
+  };
+  switch (type) {
+    case kTypeQ4K: prepare(PrepareOperands<kTypeQ4K>); break;
+    case kTypeQ5K: prepare(PrepareOperands<kTypeQ5K>); break;
+    case kTypeQ6K: prepare(PrepareOperands<kTypeQ6K>); break;
+    default: prepare(PrepareOperands<kTypeQ80>); break;
+  }
   hipError_t status = hipGetLastError();
   if (status != hipSuccess) return status;
 

@@ -247,7 +247,15 @@ int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
 /* MatMul with many tokens, the prefill shape (gguf_projections.cpp:239-286 with
  * tokens = m; NPU analogue src/npu/gemm.hpp:99-105):
  *   c[t*rows + r] = row r of w . a[t],  a given as bf16 (m x cols, row-major),
- * computed on the matrix cores with fp32 accumulation.  w must be Q4_K. */
+ * computed on the matrix cores with fp32 accumulation: both operands are converted to
+ * fp16 once per call (each weight rounded once; activations beyond +-65504 saturate).
+ * w is Q4_K, Q5_K, Q6_K or Q8_0 (MatMul takes the row type of whatever tensor the stage
+ * holds, gguf_projections.cpp:251-262); fp32 rows are GUFO_HIP_ERR_INVALID_ARGUMENT. */
+int gufo_hip_gemm_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
+                       float* c_host);
+int gufo_hip_gemm_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev, size_t m,
+                           float* c_dev);
+/* The same, refusing any w that is not Q4_K (the type of the prefill configuration). */
 int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host,
                            size_t m, float* c_host);
 int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,

@@ -90,6 +90,62 @@ def test_gemm_rejects_other_types(hip):
     with pytest.raises(hip.InvalidArgumentError):
         hip.gemm_q4k_bf16(m, np.zeros((4, 256), np.uint16))
     m.destroy()
+    f = hip.Matrix(synth.F32, synth.matrix(synth.F32, 32, 256, 2), 32, 256)
+    with pytest.raises(hip.InvalidArgumentError):
+        hip.gemm_bf16(f, np.zeros((4, 256), np.uint16))
+    f.destroy()
+
+
+OTHER_TYPES = [synth.Q5_K, synth.Q6_K, synth.Q8_0]
+
+
+@pytest.mark.parametrize("ggml_type", OTHER_TYPES)
+@pytest.mark.parametrize("tokens,rows,cols", [(128, 256, 256), (77, 200, 512), (300, 129, 2048),
+                                              (5, 33, 2304)])
+def test_gemm_parity_other_row_types(hip, oracle, ggml_type, tokens, rows, cols):
+    # The prefill product for the other row types a stage can hold: the same product
+    # kernel behind a pre-pass that dequantizes that type.
+    say("gemm", synth.TYPE_NAMES[ggml_type], tokens, rows, cols)
+    seed = 7100 + 31 * ggml_type + tokens + rows + cols
+    w = synth.matrix(ggml_type, rows, cols, seed)
+    bits, a = bf16_activations(tokens, cols, seed + 1)
+    m = hip.Matrix(ggml_type, w, rows, cols)
+    got = hip.gemm_bf16(m, bits)
+    want = oracle.matmul([(ggml_type, w, 0, rows)], a, precision="double", threads=8)
+    assert got.shape == want.shape == (tokens, rows)
+    assert oracle.rel_l2(got, want) <= TOLERANCE
+    for t in sorted({0, tokens // 2, tokens - 1}):
+        single = hip.gemv([hip.whole(m)], a[t:t + 1], 1)
+        assert oracle.rel_l2(got[t], single[0]) <= VS_GEMV
+    m.destroy()
+
+
+@pytest.mark.parametrize("ggml_type", [synth.Q5_K, synth.Q6_K])
+def test_gemm_unit_activations_return_the_weights_other_types(hip, oracle, ggml_type):
+    # Every weight of the matrix, one by one, as the pre-pass dequantized it: within half
+    # an fp16 ulp of the checker's dequantization (pinned by the reference's fixtures).
+    # A wrong bit of a code, a wrong scale index or a wrong position shows here.
+    say("gemm identity", synth.TYPE_NAMES[ggml_type])
+    rows, cols = 64, 512
+    w = synth.kquant_matrix(ggml_type, rows, cols, 98)
+    m = hip.Matrix(ggml_type, w, rows, cols)
+    bits = synth.bf16_round(np.eye(cols, dtype=np.float32))
+    got = hip.gemm_bf16(m, bits)
+    want = np.stack([oracle.dequantize(ggml_type, w[r], cols) for r in range(rows)], axis=1)
+    bound = np.maximum(np.abs(want) * 2.0 ** -11, 2.0 ** -25)
+    if ggml_type == synth.Q5_K:  # d sc q - dmin m is rounded once more, in fp32
+        bound = bound + 2.0 ** -23 * np.abs(want).max(axis=0, keepdims=True)
+    assert bool(np.all(np.abs(got.astype(np.float64) - want) <= bound))
+    m.destroy()
+
+
+def test_gemm_q4k_entry_point_equals_the_general_one(hip):
+    w = synth.kquant_matrix(synth.Q4_K, 96, 512, 5)
+    m = hip.Matrix(synth.Q4_K, w, 96, 512)
+    bits, _ = bf16_activations(40, 512, 6)
+    assert bool(np.array_equal(hip.gemm_q4k_bf16(m, bits).view(np.uint32),
+                               hip.gemm_bf16(m, bits).view(np.uint32)))
+    m.destroy()
 
 
 def test_config5_prefill_projection(hip, oracle):
