@@ -73,7 +73,8 @@ struct State {
   Scratch moe_tables;   // counts, offsets, pairs, valid flags, segments
   Scratch moe_gate_up;  // pairs x 2*ffn
   Scratch moe_out;      // pairs x hidden
-  Scratch gemm_work;    // prefill: fp16 activations + sub-block sums
+  Scratch moe_route;    // whole-layer call: router logits, then ids, then weights
+  Scratch gemm_work;    // prefill: both operands as fp16
   Scratch stage_c;      // prefill, host-pointer variant: device copy of C
 };
 
@@ -419,8 +420,8 @@ int CopyOut(void* host, const void* device, size_t bytes) {
   return GUFO_HIP_OK;
 }
 
-int RouteDevLocked(const float* logits, int tokens, int experts, int k, int* ids,
-                   float* weights) {
+int RouteDevLocked(const float* logits, size_t logit_stride, int tokens, int experts, int k,
+                   int* ids, float* weights) {
   if (tokens < 0 || k <= 0 || experts <= 0 || k > experts) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "route: tokens %d, experts %d, k %d",
                 tokens, experts, k);
@@ -431,7 +432,8 @@ int RouteDevLocked(const float* logits, int tokens, int experts, int k, int* ids
                 gufo::kMaxRouteExperts, gufo::kMaxRouteK);
   }
   if (tokens == 0) return GUFO_HIP_OK;
-  GUFO_HIP_TRY(gufo::LaunchRoute(logits, tokens, experts, k, ids, weights, g_state.stream));
+  GUFO_HIP_TRY(gufo::LaunchRoute(logits, logit_stride, tokens, experts, k, ids, weights,
+                                 g_state.stream));
   return GUFO_HIP_OK;
 }
 
@@ -466,7 +468,8 @@ int GroupDevLocked(const int* ids, int tokens, int k, int experts, bool segments
 
 int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                     const gufo_hip_matrix* down, int experts, const float* x, int tokens,
-                    const int* ids, const float* weights, int k, float* y) {
+                    const int* ids, const float* weights, int k,
+                    const gufo::MoeShared& shared, float* y) {
   if (gate == nullptr || up == nullptr || down == nullptr) {
     return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no MoE experts");
   }
@@ -570,11 +573,11 @@ int MoeFfnDevLocked(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   }
   if (direct) {
     GUFO_HIP_TRY(gufo::LaunchMoeCombineDirect(routed, weights, ids, experts, k,
-                                              static_cast<int>(hidden), y, tables.header,
-                                              g_state.stream));
+                                              static_cast<int>(hidden), shared, y,
+                                              tables.header, g_state.stream));
   } else {
     GUFO_HIP_TRY(gufo::LaunchMoeCombine(routed, weights, tables.valid, tokens, k,
-                                        static_cast<int>(hidden), y, g_state.stream));
+                                        static_cast<int>(hidden), shared, y, g_state.stream));
   }
   g_state.moe_pending = true;
   return GUFO_HIP_OK;
@@ -658,6 +661,7 @@ int gufo_hip_shutdown(void) {
   Release(&g_state.moe_tables);
   Release(&g_state.moe_gate_up);
   Release(&g_state.moe_out);
+  Release(&g_state.moe_route);
   Release(&g_state.gemm_work);
   Release(&g_state.stage_c);
   (void)hipEventDestroy(g_state.timer_begin);
@@ -923,7 +927,8 @@ int gufo_hip_route_topk_dev(const float* logits_dev, int tokens, int experts, in
                             int* ids_dev, float* weights_dev) {
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
-  return RouteDevLocked(logits_dev, tokens, experts, k, ids_dev, weights_dev);
+  return RouteDevLocked(logits_dev, static_cast<size_t>(experts > 0 ? experts : 0), tokens,
+                        experts, k, ids_dev, weights_dev);
 }
 
 int gufo_hip_route_topk(const float* logits_host, int tokens, int experts, int k,
@@ -940,8 +945,9 @@ int gufo_hip_route_topk(const float* logits_host, int tokens, int experts, int k
                   static_cast<size_t>(tokens) * experts * sizeof(float)));
   GUFO_TRY(Reserve(&g_state.stage_ids, n * sizeof(int)));
   GUFO_TRY(Reserve(&g_state.stage_weights, n * sizeof(float)));
-  GUFO_TRY(RouteDevLocked(static_cast<const float*>(g_state.stage_x.ptr), tokens, experts,
-                          k, static_cast<int*>(g_state.stage_ids.ptr),
+  GUFO_TRY(RouteDevLocked(static_cast<const float*>(g_state.stage_x.ptr),
+                          static_cast<size_t>(experts), tokens, experts, k,
+                          static_cast<int*>(g_state.stage_ids.ptr),
                           static_cast<float*>(g_state.stage_weights.ptr)));
   GUFO_TRY(CopyOut(ids_host, g_state.stage_ids.ptr, n * sizeof(int)));
   return CopyOut(weights_host, g_state.stage_weights.ptr, n * sizeof(float));
@@ -985,6 +991,53 @@ int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
   return MoeFfnDevLocked(gate, up, down, experts, x_dev, tokens, ids_dev, weights_dev, k,
+                         gufo::MoeShared{}, y_dev);
+}
+
+int gufo_hip_moe_layer_dev(const gufo_hip_matrix* router, const gufo_hip_matrix* gate,
+                           const gufo_hip_matrix* up, const gufo_hip_matrix* down, int experts,
+                           int k, const float* x_dev, int tokens, const float* shared_dev,
+                           float* y_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (router == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no router");
+  if (experts <= 0 || tokens < 0 || k <= 0 || k > experts) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: experts %d, tokens %d, k %d", experts,
+                tokens, k);
+  }
+  // The router yields one logit per expert, and one more - the shared expert's gate -
+  // when the model has a shared expert (src/models/qwen35/decoder.cpp:537-539).
+  const size_t logits = router->rows;
+  const size_t needed = static_cast<size_t>(experts) + (shared_dev != nullptr ? 1 : 0);
+  if (logits < needed || logits > static_cast<size_t>(experts) + 1) {
+    return Fail(GUFO_HIP_ERR_SHAPE,
+                "a router of %zu rows does not serve %d experts %s a shared expert", logits,
+                experts, shared_dev != nullptr ? "and" : "without");
+  }
+  if (gate != nullptr && router->cols != gate->cols) {
+    return Fail(GUFO_HIP_ERR_SHAPE, "router rows of %zu values, expert rows of %zu",
+                router->cols, gate->cols);
+  }
+  if (tokens == 0) return GUFO_HIP_OK;
+  const size_t n = static_cast<size_t>(tokens);
+  const size_t logit_bytes = Align16(n * logits * sizeof(float));
+  const size_t id_bytes = Align16(n * k * sizeof(int));
+  GUFO_TRY(Reserve(&g_state.moe_route, logit_bytes + id_bytes + n * k * sizeof(float)));
+  uint8_t* base = static_cast<uint8_t*>(g_state.moe_route.ptr);
+  float* logit = reinterpret_cast<float*>(base);
+  int* ids = reinterpret_cast<int*>(base + logit_bytes);
+  float* weights = reinterpret_cast<float*>(base + logit_bytes + id_bytes);
+  const size_t first = 0;
+  GUFO_TRY(GemvDevLocked(&router, &first, &logits, 1, gufo::GemvPrologue{}, x_dev, tokens,
+                         logit));
+  GUFO_TRY(RouteDevLocked(logit, logits, tokens, experts, k, ids, weights));
+  gufo::MoeShared shared;
+  if (shared_dev != nullptr) {
+    shared.rows = shared_dev;
+    shared.gate_logit = logit + experts;
+    shared.gate_stride = logits;
+  }
+  return MoeFfnDevLocked(gate, up, down, experts, x_dev, tokens, ids, weights, k, shared,
                          y_dev);
 }
 
@@ -1014,7 +1067,7 @@ int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                            static_cast<const float*>(g_state.stage_x.ptr), tokens,
                            static_cast<const int*>(g_state.stage_ids.ptr),
                            static_cast<const float*>(g_state.stage_weights.ptr), k,
-                           static_cast<float*>(g_state.stage_y.ptr)));
+                           gufo::MoeShared{}, static_cast<float*>(g_state.stage_y.ptr)));
   GUFO_TRY(CopyOut(y_host, g_state.stage_y.ptr, tokens * hidden * sizeof(float)));
   return CheckMoeIdsLocked();
 }

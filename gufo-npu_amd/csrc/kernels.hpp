@@ -127,11 +127,20 @@ hipError_t LaunchMoeGemv(int type, const GemvLaunch& launch, const MoeGemvArgs& 
                          bool swiglu, uint32_t max_segments, int max_pairs,
                          hipStream_t stream);
 
-// Softmax (double) top-k routing of `tokens` rows of `experts` logits.
+// Softmax (double) top-k routing of `tokens` rows of `experts` logits, the rows
+// logit_stride floats apart (a router with a shared-expert gate yields experts + 1).
 constexpr int kMaxRouteExperts = 1024;
 constexpr int kMaxRouteK = 64;
-hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int* ids,
-                       float* weights, hipStream_t stream);
+hipError_t LaunchRoute(const float* logits, size_t logit_stride, int tokens, int experts, int k,
+                       int* ids, float* weights, hipStream_t stream);
+
+// The shared expert's contribution to a combine: its output rows (tokens x hidden; null:
+// none) and each token's gate logit (gate_stride floats apart).
+struct MoeShared {
+  const float* rows = nullptr;
+  const float* gate_logit = nullptr;
+  size_t gate_stride = 0;
+};
 
 // Groups the n_pairs = tokens*k pairs by expert: counts[experts],
 // offsets[experts+1], pairs[n_pairs] (ascending pair id within an expert),
@@ -152,17 +161,18 @@ hipError_t LaunchMoeGroupSmall(const int* ids, int n_pairs, int experts, int cap
                                hipStream_t stream);
 
 // y[t][i] = sum over slots in order of weights[t*k+slot] * rows[(t*k+slot)][i],
-// accumulated in double; invalid pairs are skipped.
+// accumulated in double; invalid pairs are skipped.  With shared.rows the sum starts from
+// shared.rows[t][i] * sigmoid(gate logit of t); y may then be shared.rows itself.
 hipError_t LaunchMoeCombine(const float* rows, const float* weights,
                             const uint8_t* pair_valid, int tokens, int k, int hidden,
-                            float* y, hipStream_t stream);
+                            const MoeShared& shared, float* y, hipStream_t stream);
 
 // The same for one token whose pairs were not grouped: a slot is valid when its id is
 // below `experts`; also fills *tables from the ids (what the grouping kernel would have
 // written), so that out-of-range ids are reported as after a grouped call.
 hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const int32_t* ids,
-                                  int experts, int k, int hidden, float* y, MoeTables* tables,
-                                  hipStream_t stream);
+                                  int experts, int k, int hidden, const MoeShared& shared,
+                                  float* y, MoeTables* tables, hipStream_t stream);
 
 // ---- prefill ------------------------------------------------------------------
 

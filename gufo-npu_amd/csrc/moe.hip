@@ -38,7 +38,8 @@ __device__ __forceinline__ int Precedes(double other, int other_index, double mi
 }
 
 __global__ __launch_bounds__(kRouteThreads) void RouteKernel(
-    const float* __restrict__ logits, int experts, int k, int* ids, float* weights) {
+    const float* __restrict__ logits, size_t logit_stride, int experts, int k, int* ids,
+    float* weights) {
   __shared__ __align__(16) double lds_prob[kMaxRouteExperts];
   __shared__ __align__(16) double lds_survivor[kMaxRouteExperts];
   __shared__ int lds_survivor_index[kMaxRouteExperts];
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(kRouteThreads) void RouteKernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const float* row = logits + static_cast<size_t>(blockIdx.x) * experts;
+  const float* row = logits + static_cast<size_t>(blockIdx.x) * logit_stride;
   const int padded = (experts + kRouteChunk - 1) / kRouteChunk * kRouteChunk;
 
   float logit[kRoutePerThread];
@@ -331,13 +332,25 @@ __global__ __launch_bounds__(64) void MoeGroupSmallKernel(
 // out[t][i] = sum over slots in slot order of weight * routed row, in double
 // (src/models/qwen35/reference.cpp:595-606 of the reference).  One fixed order,
 // no atomics: repeated runs give identical bits.
+//
+// With a shared expert the sum starts from its output times SharedExpertScale of the
+// token's gate logit, sigmoid in double rounded to fp32, the product in fp32
+// (src/models/qwen35/moe.cpp:44-47, decoder.cpp:539-542).
+__device__ __forceinline__ double SharedTerm(const MoeShared& shared, int t, int hidden, int i) {
+  if (shared.rows == nullptr) return 0.0;
+  const double logit = static_cast<double>(shared.gate_logit[static_cast<size_t>(t) * shared.gate_stride]);
+  const float scale = static_cast<float>(1.0 / (1.0 + exp(-logit)));
+  return static_cast<double>(shared.rows[static_cast<size_t>(t) * hidden + i] * scale);
+}
+
 __global__ __launch_bounds__(256) void MoeCombineKernel(
     const float* __restrict__ rows, const float* __restrict__ weights,
-    const uint8_t* __restrict__ pair_valid, int k, int hidden, float* __restrict__ y) {
+    const uint8_t* __restrict__ pair_valid, int k, int hidden, const MoeShared shared,
+    float* y) {  // may be shared.rows: every thread reads its element before writing it
   const int t = blockIdx.y;
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= hidden) return;
-  double acc = 0.0;
+  double acc = SharedTerm(shared, t, hidden, i);
   for (int slot = 0; slot < k; ++slot) {
     const size_t s = static_cast<size_t>(t) * k + slot;
     if (pair_valid[s] == 0) continue;
@@ -350,8 +363,8 @@ __global__ __launch_bounds__(256) void MoeCombineKernel(
 // the launch writes the header the grouping kernel would have written.
 __global__ __launch_bounds__(256) void MoeCombineDirectKernel(
     const float* __restrict__ rows, const float* __restrict__ weights,
-    const int32_t* __restrict__ ids, int experts, int k, int hidden, float* __restrict__ y,
-    MoeTables* tables) {
+    const int32_t* __restrict__ ids, int experts, int k, int hidden, const MoeShared shared,
+    float* y, MoeTables* tables) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i == 0) {
     int invalid = 0;
@@ -372,7 +385,7 @@ __global__ __launch_bounds__(256) void MoeCombineDirectKernel(
     tables->pad = 0;
   }
   if (i >= hidden) return;
-  double acc = 0.0;
+  double acc = SharedTerm(shared, 0, hidden, i);
   for (int slot = 0; slot < k; ++slot) {
     const int e = ids[slot];
     if (e < 0 || e >= experts) continue;
@@ -385,23 +398,23 @@ __global__ __launch_bounds__(256) void MoeCombineDirectKernel(
 }  // namespace
 
 hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const int32_t* ids,
-                                  int experts, int k, int hidden, float* y, MoeTables* tables,
-                                  hipStream_t stream) {
+                                  int experts, int k, int hidden, const MoeShared& shared,
+                                  float* y, MoeTables* tables, hipStream_t stream) {
   if (hidden <= 0 || k <= 0) return hipErrorInvalidValue;
   hipLaunchKernelGGL(MoeCombineDirectKernel, dim3((hidden + 255) / 256), dim3(256), 0, stream,
-                     rows, weights, ids, experts, k, hidden, y, tables);
+                     rows, weights, ids, experts, k, hidden, shared, y, tables);
   return hipGetLastError();
 }
 
-hipError_t LaunchRoute(const float* logits, int tokens, int experts, int k, int* ids,
-                       float* weights, hipStream_t stream) {
+hipError_t LaunchRoute(const float* logits, size_t logit_stride, int tokens, int experts, int k,
+                       int* ids, float* weights, hipStream_t stream) {
   if (tokens < 0 || experts < 1 || experts > kMaxRouteExperts || k < 1 ||
-      k > kMaxRouteK || k > experts) {
+      k > kMaxRouteK || k > experts || logit_stride < static_cast<size_t>(experts)) {
     return hipErrorInvalidValue;
   }
   if (tokens == 0) return hipSuccess;
   hipLaunchKernelGGL(RouteKernel, dim3(tokens), dim3(kRouteThreads), 0, stream, logits,
-                     experts, k, ids, weights);
+                     logit_stride, experts, k, ids, weights);
   return hipGetLastError();
 }
 
@@ -432,10 +445,10 @@ hipError_t LaunchMoeGroupSmall(const int* ids, int n_pairs, int experts, int cap
 
 hipError_t LaunchMoeCombine(const float* rows, const float* weights,
                             const uint8_t* pair_valid, int tokens, int k, int hidden,
-                            float* y, hipStream_t stream) {
+                            const MoeShared& shared, float* y, hipStream_t stream) {
   if (tokens <= 0 || hidden <= 0) return hipSuccess;
   hipLaunchKernelGGL(MoeCombineKernel, dim3((hidden + 255) / 256, tokens), dim3(256), 0,
-                     stream, rows, weights, pair_valid, k, hidden, y);
+                     stream, rows, weights, pair_valid, k, hidden, shared, y);
   return hipGetLastError();
 }
 

@@ -288,6 +288,33 @@ def swiglu(gate_up: np.ndarray) -> np.ndarray:
     return act
 
 
+def shared_expert_scale(logit, use_ref: bool = False) -> np.float32:
+    """Sigmoid of the shared expert's gate logit, in double, rounded to fp32
+    (models/qwen35/moe.cpp:44-47)."""
+    if use_ref:
+        return np.float32(ref().ref_shared_expert_scale(float(np.float32(logit))))
+    return np.float32(1.0 / (1.0 + np.exp(-np.float64(np.float32(logit)))))
+
+
+def moe_layer(router_type, router, gate, gate_type, up, up_type, down, down_type, experts,
+              hidden, ffn, x, k, shared=None, threads: int = 1):
+    """Decoder::MoeFfn (models/qwen35/decoder.cpp:530-558) for every token of x: the router
+    product, Route over its first `experts` logits, the chosen experts, and - with
+    `shared`, the shared expert's output rows - the start value shared * scale(logit
+    `experts`).  Products and sums in double.  Returns ids, weights, y."""
+    x = _f32(x)
+    rows = router.shape[0]
+    logits = matmul([(router_type, router, 0, rows)], x, precision="double", threads=threads)
+    ids, weights, routed = moe_ffn(gate, gate_type, up, up_type, down, down_type, experts,
+                                   hidden, ffn, np.ascontiguousarray(logits[:, :experts]), x, k,
+                                   precision="double", threads=threads)
+    y = routed.astype(np.float64)
+    if shared is not None:
+        scale = np.array([shared_expert_scale(l) for l in logits[:, experts]], np.float32)
+        y = y + (_f32(shared) * scale[:, None]).astype(np.float64)
+    return ids, weights, y.astype(np.float32)
+
+
 CONFIG_FIELDS = ("layers", "mtp_layers", "hidden", "ffn", "vocab", "full_attention_interval",
                  "heads", "kv_heads", "head_dim", "rope_dim", "conv_kernel", "linear_key_heads",
                  "linear_value_heads", "linear_head_dim", "experts", "experts_used",

@@ -39,6 +39,7 @@ class Sequence:
         self.up = make(synth.Q4_K, ffn, hidden, 2)
         self.down = make(synth.Q6_K, hidden, ffn, 3)
         self.router = make(synth.F32, experts, hidden, 4)
+        self.router_gate = make(synth.F32, experts + 1, hidden, 10)
         self.gate_exps = make(synth.Q4_K, experts * expert_ffn, hidden, 5)
         self.up_exps = make(synth.Q4_K, experts * expert_ffn, hidden, 6)
         self.down_exps = make(synth.Q5_K, experts * hidden, expert_ffn, 7)
@@ -49,7 +50,7 @@ class Sequence:
         f = lambda n: hip.DeviceBuffer(4 * tokens * n)
         self.h, self.delta, self.h1, self.normed = f(hidden), f(hidden), f(hidden), f(hidden)
         self.gate_up, self.ffn_out = f(2 * ffn), f(hidden)
-        self.logits, self.moe_out = f(experts), f(hidden)
+        self.logits, self.moe_out, self.layer_out = f(experts), f(hidden), f(hidden)
         self.ids, self.weights = hip.DeviceBuffer(4 * tokens * 4), hip.DeviceBuffer(4 * tokens * 4)
         self.token = hip.DeviceBuffer(8 * tokens)
         self.a16 = hip.DeviceBuffer(2 * 64 * hidden)
@@ -72,6 +73,9 @@ class Sequence:
         hip.route_topk_dev(self.logits, n, s["experts"], s["k"], self.ids, self.weights)
         hip.moe_ffn_dev(self.gate_exps, self.up_exps, self.down_exps, s["experts"], self.normed,
                         n, self.ids, self.weights, s["k"], self.moe_out)
+        # the whole mixture layer in one call, over the dense FFN's output as shared expert
+        hip.moe_layer_dev(self.router_gate, self.gate_exps, self.up_exps, self.down_exps,
+                          s["experts"], s["k"], self.normed, n, self.ffn_out, self.layer_out)
         hip.gemv_argmax_dev([hip.whole(self.head)],
                             hip.resnorm_prologue(self.norm, EPS, self.ffn_out), self.h1, n,
                             self.token)
@@ -87,12 +91,14 @@ class Sequence:
             "ids": self.ids.download((n, s["k"]), np.int32),
             "weights": self.weights.download((n, s["k"]), np.float32),
             "moe_out": self.moe_out.download((n, s["hidden"]), np.float32),
+            "layer_out": self.layer_out.download((n, s["hidden"]), np.float32),
             "token": self.token.download((n,), np.int64),
             "c": self.c.download((64, 256), np.float32),
         }
 
     def clear_outputs(self):
         for b in (self.h1, self.normed, self.gate_up, self.ffn_out, self.logits, self.moe_out,
+                  self.layer_out,
                   self.ids, self.weights, self.token, self.c):
             b.upload(np.zeros(b.nbytes, dtype=np.uint8))
 

@@ -423,3 +423,45 @@ def test_moe_ffn_equals_per_token_result(oracle):
             out = oracle.matmul([(synth.Q5_K, down, e * hidden, hidden)], act[None, :])[0]
             acc += np.float64(weights[t, slot]) * out.astype(np.float64)
         assert np.array_equal(y[t], acc.astype(np.float32))
+
+
+def test_shared_expert_scale_is_the_sigmoid(oracle):
+    # Closed forms: 1/2 at 0, s(v) + s(-v) = 1, saturation, and the textbook value at 1.
+    assert oracle.shared_expert_scale(0.0) == np.float32(0.5)
+    assert oracle.shared_expert_scale(1.0) == np.float32(1.0 / (1.0 + math.exp(-1.0)))
+    assert oracle.shared_expert_scale(200.0) == np.float32(1.0)
+    assert oracle.shared_expert_scale(-200.0) == np.float32(0.0)
+    for v in synth.router_logits(1, 64, 77)[0] * np.float32(4.0):
+        total = np.float64(oracle.shared_expert_scale(v)) + np.float64(oracle.shared_expert_scale(-v))
+        assert abs(total - 1.0) <= 2.0 ** -24
+
+
+def test_shared_expert_scale_equals_the_compiled_reference(ref_oracle):
+    for v in np.concatenate([synth.router_logits(1, 256, 78)[0] * np.float32(6.0),
+                             np.array([0.0, -0.0, 88.0, -88.0, 1e-30], np.float32)]):
+        assert ref_oracle.shared_expert_scale(v) == ref_oracle.shared_expert_scale(v, use_ref=True)
+
+
+def test_moe_layer_is_router_plus_routed_experts_plus_scaled_shared_expert(oracle):
+    experts, hidden, ffn, k, tokens = 8, 256, 256, 2, 3
+    router = synth.f32_matrix(experts + 1, hidden, 60)
+    gate = synth.kquant_matrix(synth.Q4_K, experts * ffn, hidden, 61)
+    up = synth.kquant_matrix(synth.Q4_K, experts * ffn, hidden, 62)
+    down = synth.kquant_matrix(synth.Q6_K, experts * hidden, ffn, 63)
+    x = synth.activations(tokens, hidden, 64) * np.float32(0.05)
+    shared = synth.activations(tokens, hidden, 65)
+    ids, weights, y = oracle.moe_layer(synth.F32, router, gate, synth.Q4_K, up, synth.Q4_K, down,
+                                       synth.Q6_K, experts, hidden, ffn, x, k, shared=shared)
+    w = router.view(np.float32).reshape(experts + 1, hidden).astype(np.float64)
+    logits = (x.astype(np.float64) @ w.T).astype(np.float32)
+    want_ids, want_w = oracle.route(np.ascontiguousarray(logits[:, :experts]), k)
+    assert np.array_equal(ids, want_ids) and np.allclose(weights, want_w, rtol=1e-6)
+    _, _, routed = oracle.moe_ffn(gate, synth.Q4_K, up, synth.Q4_K, down, synth.Q6_K, experts,
+                                  hidden, ffn, np.ascontiguousarray(logits[:, :experts]), x, k,
+                                  precision="double")
+    _, _, without = oracle.moe_layer(synth.F32, router, gate, synth.Q4_K, up, synth.Q4_K, down,
+                                     synth.Q6_K, experts, hidden, ffn, x, k)
+    assert oracle.rel_l2(without, routed) <= 1e-7
+    for t in range(tokens):
+        scale = 1.0 / (1.0 + math.exp(-float(logits[t, experts])))
+        assert oracle.rel_l2(y[t], routed[t].astype(np.float64) + scale * shared[t]) <= 1e-6
