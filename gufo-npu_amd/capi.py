@@ -100,7 +100,8 @@ SIGNATURES = {
     "gufo_hip_moe_ffn": (C.c_int, [_P, _P, _P, C.c_int, _P, C.c_int, _P, _P, C.c_int, _P]),
     "gufo_hip_moe_ffn_dev": (C.c_int, [_P, _P, _P, C.c_int, _P, C.c_int, _P, _P, C.c_int,
                                        _P]),
-    "gufo_hip_moe_layer_dev": (C.c_int, [_P, _P, _P, _P, C.c_int, C.c_int, _P, C.c_int, _P, _P]),
+    "gufo_hip_moe_layer_dev": (C.c_int, [_P, C.c_int, _P, _P, _P, C.c_int, C.c_int, _P, C.c_int,
+                                         _P, _P]),
     "gufo_hip_gemm_bf16": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_bf16_dev": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_q4k_bf16": (C.c_int, [_P, _P, _SZ, _P]),
@@ -386,13 +387,15 @@ def moe_ffn_dev(gate: Matrix, up: Matrix, down: Matrix, experts: int, x: DeviceB
         C.c_void_p(y.ptr)))
 
 
-def moe_layer_dev(router: Matrix, gate: Matrix, up: Matrix, down: Matrix, experts: int, k: int,
-                  x: DeviceBuffer, tokens: int, shared: "DeviceBuffer | None",
-                  y: DeviceBuffer) -> None:
+def moe_layer_dev(router: "Matrix | Sequence[Matrix]", gate: Matrix, up: Matrix, down: Matrix,
+                  experts: int, k: int, x: DeviceBuffer, tokens: int,
+                  shared: "DeviceBuffer | None", y: DeviceBuffer) -> None:
     """Router, routing, routed experts and the scaled shared expert in one call
-    (gufo_hip_moe_layer_dev)."""
+    (gufo_hip_moe_layer_dev).  `router`: the matrix, or the matrices, of the router stage."""
+    parts = [router] if isinstance(router, Matrix) else list(router)
+    handles = (C.c_void_p * len(parts))(*[m.handle for m in parts])
     _check(load_library().gufo_hip_moe_layer_dev(
-        C.c_void_p(router.handle), C.c_void_p(gate.handle), C.c_void_p(up.handle),
+        handles, len(parts), C.c_void_p(gate.handle), C.c_void_p(up.handle),
         C.c_void_p(down.handle), experts, k, C.c_void_p(x.ptr), tokens, _dev_ptr(shared),
         C.c_void_p(y.ptr)))
 

@@ -994,29 +994,42 @@ int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                          gufo::MoeShared{}, y_dev);
 }
 
-int gufo_hip_moe_layer_dev(const gufo_hip_matrix* router, const gufo_hip_matrix* gate,
-                           const gufo_hip_matrix* up, const gufo_hip_matrix* down, int experts,
-                           int k, const float* x_dev, int tokens, const float* shared_dev,
+int gufo_hip_moe_layer_dev(const gufo_hip_matrix* const* router_parts, int n_router_parts,
+                           const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                           const gufo_hip_matrix* down, int experts, int k,
+                           const float* x_dev, int tokens, const float* shared_dev,
                            float* y_dev) {
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
-  if (router == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no router");
+  if (router_parts == nullptr || n_router_parts < 1 || n_router_parts > kMaxGemvParts) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no router");
+  }
   if (experts <= 0 || tokens < 0 || k <= 0 || k > experts) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "moe: experts %d, tokens %d, k %d", experts,
                 tokens, k);
   }
-  // The router yields one logit per expert, and one more - the shared expert's gate -
-  // when the model has a shared expert (src/models/qwen35/decoder.cpp:537-539).
-  const size_t logits = router->rows;
+  // The router stage yields one logit per expert, and one more - the shared expert's
+  // gate, a tensor of its own - when the model has a shared expert
+  // (src/models/qwen35/gguf_projections.cpp:127-131, decoder.cpp:537-539).
+  size_t first_rows[kMaxGemvParts] = {0};
+  size_t part_rows[kMaxGemvParts] = {0};
+  size_t logits = 0;
+  for (int p = 0; p < n_router_parts; ++p) {
+    if (router_parts[p] == nullptr) {
+      return Fail(GUFO_HIP_ERR_LOGIC, "these projections have no router");
+    }
+    part_rows[p] = router_parts[p]->rows;
+    logits += part_rows[p];
+  }
   const size_t needed = static_cast<size_t>(experts) + (shared_dev != nullptr ? 1 : 0);
   if (logits < needed || logits > static_cast<size_t>(experts) + 1) {
     return Fail(GUFO_HIP_ERR_SHAPE,
                 "a router of %zu rows does not serve %d experts %s a shared expert", logits,
                 experts, shared_dev != nullptr ? "and" : "without");
   }
-  if (gate != nullptr && router->cols != gate->cols) {
+  if (gate != nullptr && router_parts[0]->cols != gate->cols) {
     return Fail(GUFO_HIP_ERR_SHAPE, "router rows of %zu values, expert rows of %zu",
-                router->cols, gate->cols);
+                router_parts[0]->cols, gate->cols);
   }
   if (tokens == 0) return GUFO_HIP_OK;
   const size_t n = static_cast<size_t>(tokens);
@@ -1027,9 +1040,8 @@ int gufo_hip_moe_layer_dev(const gufo_hip_matrix* router, const gufo_hip_matrix*
   float* logit = reinterpret_cast<float*>(base);
   int* ids = reinterpret_cast<int*>(base + logit_bytes);
   float* weights = reinterpret_cast<float*>(base + logit_bytes + id_bytes);
-  const size_t first = 0;
-  GUFO_TRY(GemvDevLocked(&router, &first, &logits, 1, gufo::GemvPrologue{}, x_dev, tokens,
-                         logit));
+  GUFO_TRY(GemvDevLocked(router_parts, first_rows, part_rows, n_router_parts,
+                         gufo::GemvPrologue{}, x_dev, tokens, logit));
   GUFO_TRY(RouteDevLocked(logit, logits, tokens, experts, k, ids, weights));
   gufo::MoeShared shared;
   if (shared_dev != nullptr) {

@@ -317,4 +317,17 @@ void HipProjections::RoutedFfn(int layer, const float* x, int tokens, const int*
                          tokens, chosen, weights, k, y));
 }
 
+void HipProjections::MoeLayerDevice(int layer, const float* x, int tokens, int k,
+                                    const float* shared, float* y) const {
+  const Layer& l = layers_.at(static_cast<std::size_t>(layer));
+  if (l.gate_exps.handle == nullptr || l.router.empty()) {
+    throw std::logic_error("qwen35: these projections have no MoE experts");
+  }
+  std::vector<const gufo_hip_matrix*> router;
+  for (const Matrix& m : l.router) router.push_back(m.handle);
+  Check(gufo_hip_moe_layer_dev(router.data(), static_cast<int>(router.size()),
+                               l.gate_exps.handle, l.up_exps.handle, l.down_exps.handle,
+                               experts_, k, x, tokens, shared, y));
+}
+
 }  // namespace gufo_hip

@@ -145,6 +145,12 @@ public:
   // shared expert.  Tokens are grouped by expert on the device.
   void RoutedFfn(int layer, const float* x, int tokens, const int* chosen, const float* weights,
                  int k, float* y) const;
+  // Decoder::MoeFfn whole on rows in device memory (decoder.cpp:530-558): the kRouter
+  // product of x, Route, the k chosen experts and, with `shared` (the shared expert's
+  // output, tokens x hidden; y may be the same rows), shared * SharedExpertScale of the
+  // router's last logit as the start of the sum.  Enqueued, not waited for.
+  void MoeLayerDevice(int layer, const float* x, int tokens, int k, const float* shared,
+                      float* y) const;
 
 private:
   struct Matrix {

@@ -474,6 +474,63 @@ void RunPick(std::mt19937& rng) {
   }
 }
 
+// Decoder::MoeFfn in one call on device rows (src/models/qwen35/decoder.cpp:530-558)
+// against the same steps through the host-pointer methods: the kRouter product (two
+// tensors: the experts' rows and the shared expert's gate row), Route, RoutedFfn, and the
+// shared expert's rows scaled by the sigmoid of the last logit.
+void RunMoeLayer(std::mt19937& rng) {
+  const int experts = 8, top = 3;
+  const std::size_t hidden = 512, ffn = 256;
+  const Weights gate = RandomWeights(GUFO_ORACLE_Q4_K, experts * ffn, hidden, rng);
+  const Weights up = RandomWeights(GUFO_ORACLE_Q4_K, experts * ffn, hidden, rng);
+  const Weights down = RandomWeights(GUFO_ORACLE_Q6_K, experts * hidden, ffn, rng);
+  const Weights router = RandomWeights(GUFO_ORACLE_Q5_K, experts, hidden, rng);
+  const Weights shared_gate = RandomWeights(GUFO_ORACLE_Q5_K, 1, hidden, rng);
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  model.experts = experts;
+  model.expert_ffn = static_cast<int>(ffn);
+  LayerTensors layer;
+  layer.gate_exps = AsTensor("blk.0.ffn_gate_exps.weight", gate, experts);
+  layer.up_exps = AsTensor("blk.0.ffn_up_exps.weight", up, experts);
+  layer.down_exps = AsTensor("blk.0.ffn_down_exps.weight", down, experts);
+  layer.router = {AsTensor("blk.0.ffn_gate_inp.weight", router),
+                  AsTensor("blk.0.ffn_gate_inp_shexp.weight", shared_gate)};
+  model.layers.push_back(layer);
+  const HipProjections proj(model);
+
+  for (const int tokens : {1, 5}) {
+    const auto n = static_cast<std::size_t>(tokens);
+    const auto x = RandomActivations(n * hidden, rng, 0.02f);
+    const auto shared = RandomActivations(n * hidden, rng, 100.0f);
+    std::vector<float> logits(n * (experts + 1)), routing(n * experts);
+    proj.Apply(Stage::kRouter, 0, x.data(), tokens, logits.data());
+    for (std::size_t t = 0; t < n; ++t) {
+      std::copy_n(&logits[t * (experts + 1)], experts, &routing[t * experts]);
+    }
+    std::vector<int> chosen(n * top);
+    std::vector<float> weights(n * top), routed(n * hidden), want(n * hidden);
+    proj.Route(routing.data(), tokens, top, chosen.data(), weights.data());
+    proj.RoutedFfn(0, x.data(), tokens, chosen.data(), weights.data(), top, routed.data());
+    for (std::size_t t = 0; t < n; ++t) {
+      const double logit = logits[t * (experts + 1) + experts];
+      const auto scale = static_cast<float>(1.0 / (1.0 + std::exp(-logit)));
+      for (std::size_t i = 0; i < hidden; ++i) {
+        want[t * hidden + i] = static_cast<float>(
+            static_cast<double>(shared[t * hidden + i] * scale) + routed[t * hidden + i]);
+      }
+    }
+    const DeviceRows d_x(x), d_shared(shared), d_y(n * hidden);
+    proj.MoeLayerDevice(0, d_x.get(), tokens, top, d_shared.get(), d_y.get());
+    const std::string tag = " tokens=" + std::to_string(tokens);
+    double err = RelL2(d_y.Download(), want);
+    Report("MoeLayerDevice with a shared expert" + tag, err <= 1e-6, err);
+    proj.MoeLayerDevice(0, d_x.get(), tokens, top, nullptr, d_y.get());
+    err = RelL2(d_y.Download(), routed);
+    Report("MoeLayerDevice without one equals RoutedFfn" + tag, err == 0.0, err);
+  }
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -482,6 +539,7 @@ int main(int argc, char** argv) {
   try {
     RunDense(rng);
     RunMoe(rng);
+    RunMoeLayer(rng);
     RunDeviceChain(rng);
     RunPick(rng);
   } catch (const std::exception& e) {

@@ -243,16 +243,19 @@ int gufo_hip_moe_ffn_dev(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
                          const float* weights_dev, int k, float* y_dev);
 
 /* Decoder::MoeFfn whole, for device-resident callers (src/models/qwen35/decoder.cpp:530-558):
- * the router product (Stage::kRouter), Route over its first `experts` logits
- * (moe.cpp:16-42), the k chosen experts of every token and their weighted sum.  With
- * shared_dev (tokens x hidden, the shared expert's output) the router must have
- * experts + 1 rows, and the sum starts from shared_dev[t] * SharedExpertScale(logit
- * `experts` of token t) (moe.cpp:44-47: sigmoid in double; decoder.cpp:539-542).
- * y_dev may be shared_dev.  Five or six launches, all recordable. */
-int gufo_hip_moe_layer_dev(const gufo_hip_matrix* router, const gufo_hip_matrix* gate,
-                           const gufo_hip_matrix* up, const gufo_hip_matrix* down,
-                           int experts, int k, const float* x_dev, int tokens,
-                           const float* shared_dev, float* y_dev);
+ * the router product (Stage::kRouter: the whole matrices router_parts[0..n), their
+ * outputs side by side as the stage's parts are, gguf_projections.cpp:127-131), Route
+ * over its first `experts` logits (moe.cpp:16-42), the k chosen experts of every token
+ * and their weighted sum.  With shared_dev (tokens x hidden, the shared expert's output)
+ * the router parts must have experts + 1 rows together, and the sum starts from
+ * shared_dev[t] * SharedExpertScale(logit `experts` of token t) (moe.cpp:44-47: sigmoid
+ * in double; decoder.cpp:539-542).  y_dev may be shared_dev.  Five to seven launches,
+ * all recordable. */
+int gufo_hip_moe_layer_dev(const gufo_hip_matrix* const* router_parts, int n_router_parts,
+                           const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
+                           const gufo_hip_matrix* down, int experts, int k,
+                           const float* x_dev, int tokens, const float* shared_dev,
+                           float* y_dev);
 
 /* ---- prefill --------------------------------------------------------------- */
 

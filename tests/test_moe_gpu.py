@@ -237,5 +237,12 @@ def test_moe_layer_in_one_call(hip, oracle, router_type, tokens):
     hip.moe_layer_dev(plain, mg, mu, md, experts, k, dx, tokens, None, dy)
     hip.synchronize()
     assert same(dy.download((tokens, hidden), np.float32), routed)
-    for m in (mr, mg, mu, md, plain):
+    # The router stage as a model file holds it: the experts' rows and the shared
+    # expert's gate row as two tensors.
+    gate_row = hip.Matrix(router_type, router[experts:], 1, hidden)
+    ds.upload(shared)  # the call in place has overwritten it
+    hip.moe_layer_dev([plain, gate_row], mg, mu, md, experts, k, dx, tokens, ds, dy)
+    hip.synchronize()
+    assert same(dy.download((tokens, hidden), np.float32), got)
+    for m in (mr, mg, mu, md, plain, gate_row):
         m.destroy()
