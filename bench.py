@@ -366,7 +366,26 @@ def run_details(capi, cfg, synth, decode, args):
                f"{'' if tokens == 1 else 'group, '}gate|up, down, combine)")
         for b in keep:
             b.free()
-    for m in (mg, mu, md):
+    # The whole layer in one call: router product (F32, 256 + 1 rows), routing, experts, and
+    # the shared expert's rows scaled by the sigmoid of the extra logit.
+    router = capi.Matrix(synth.F32, synth.f32_matrix(cfg.EXPERTS4 + 1, cfg.HIDDEN4, 990),
+                         cfg.EXPERTS4 + 1, cfg.HIDDEN4)
+    for tokens in (1, 4):
+        calls, keep = [], []
+        for r in range(16):
+            xh = synth.activations(tokens, cfg.HIDDEN4, 960 + r) * np.float32(cfg.CONFIG4_X_SCALE)
+            dx = capi.DeviceBuffer.from_array(xh)
+            shared = capi.DeviceBuffer.from_array(synth.activations(tokens, cfg.HIDDEN4, 970 + r))
+            yo = capi.DeviceBuffer(4 * tokens * cfg.HIDDEN4)
+            keep += [dx, shared, yo]
+            calls.append(lambda dx=dx, shared=shared, yo=yo: capi.moe_layer_dev(
+                router, mg, mu, md, cfg.EXPERTS4, cfg.TOPK4, dx, tokens, shared, yo))
+        ms = time_recorded(capi, calls)
+        log(f"  whole layer in one call, batch {tokens}                 {ms * 1e3:8.2f} us  "
+            f"(router product + the kernels above + the scaled shared expert in the combine)")
+        for b in keep:
+            b.free()
+    for m in (mg, mu, md, router):
         m.destroy()
 
 
