@@ -92,6 +92,7 @@ SIGNATURES = {
     "gufo_hip_gemv_argmax_dev": (C.c_int, [C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ),
                                            C.c_int, _P, _P, C.c_int, _P]),
     "gufo_hip_matrix_gather_rows": (C.c_int, [_P, _P, _SZ, C.POINTER(_P)]),
+    "gufo_hip_matrix_prepare_prefill": (C.c_int, [_P]),
     "gufo_hip_argmax_dev": (C.c_int, [_P, _SZ, C.POINTER(C.c_int64)]),
     "gufo_hip_route_topk": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
     "gufo_hip_route_topk_dev": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, _P]),
@@ -247,6 +248,10 @@ class Matrix:
         picked.handle = handle.value
         picked.nbytes = self.nbytes // max(self.rows, 1) * int(ids.size)
         return picked
+
+    def prepare_prefill(self) -> None:
+        """Keeps the weights in the prefill product's own form beside the packed rows."""
+        _check(load_library().gufo_hip_matrix_prepare_prefill(C.c_void_p(self.handle)))
 
     def destroy(self) -> None:
         if self.handle:

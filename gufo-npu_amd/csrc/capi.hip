@@ -21,6 +21,9 @@ struct gufo_hip_matrix {
   size_t row_bytes;
   size_t bytes;
   uint8_t* data;  // device
+  // The weights as fp16 fragments for the prefill product, once
+  // gufo_hip_matrix_prepare_prefill has been called (device; null before).
+  void* prefill_fragments = nullptr;
 };
 
 struct gufo_hip_graph {
@@ -796,9 +799,42 @@ int gufo_hip_matrix_destroy(gufo_hip_matrix* m) {
   if (m == nullptr) return GUFO_HIP_OK;
   GUFO_TRY(RequireReady());
   GUFO_HIP_TRY(hipStreamSynchronize(g_state.stream));
+  if (m->prefill_fragments != nullptr) GUFO_HIP_TRY(hipFree(m->prefill_fragments));
   GUFO_HIP_TRY(hipFree(m->data));
   delete m;
   --g_state.live_matrices;
+  return GUFO_HIP_OK;
+}
+
+int gufo_hip_matrix_prepare_prefill(gufo_hip_matrix* m) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  if (m == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
+  if (!gufo::GemmTakesType(m->type)) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                "the prefill GEMM takes Q4_K, Q5_K, Q6_K or Q8_0 weights; this matrix has "
+                "ggml type %d",
+                m->type);
+  }
+  if (m->prefill_fragments != nullptr || m->rows == 0) return GUFO_HIP_OK;
+  if (g_state.capturing) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "a matrix cannot be prepared while recording");
+  }
+  const uint32_t nb = static_cast<uint32_t>(m->cols / gufo::kSuperBlock);
+  const size_t bytes = gufo::GemmWeightBytes(static_cast<uint32_t>(m->rows), nb);
+  void* fragments = nullptr;
+  const hipError_t status = hipMalloc(&fragments, bytes);
+  if (status != hipSuccess) {
+    return Fail(GUFO_HIP_ERR_OUT_OF_MEMORY, "hipMalloc of %zu bytes: %s", bytes,
+                hipGetErrorString(status));
+  }
+  const hipError_t launched = gufo::LaunchGemmPrepareWeights(
+      m->type, m->data, static_cast<uint32_t>(m->rows), nb, fragments, g_state.stream);
+  if (launched != hipSuccess) {
+    (void)hipFree(fragments);
+    return Fail(GUFO_HIP_ERR_RUNTIME, "pre-pass: %s", hipGetErrorString(launched));
+  }
+  m->prefill_fragments = fragments;
   return GUFO_HIP_OK;
 }
 
@@ -863,6 +899,7 @@ int gufo_hip_matrix_gather_rows(const gufo_hip_matrix* src, const int64_t* rows_
   m->rows = n;
   m->bytes = n * src->row_bytes;
   m->data = nullptr;
+  m->prefill_fragments = nullptr;  // the source's are its own
   hipError_t status = hipMalloc(reinterpret_cast<void**>(&m->data), m->bytes + 64);
   if (status != hipSuccess) {
     delete m;
@@ -1106,9 +1143,14 @@ int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* 
   if (m > (1ull << 24)) {
     return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens exceed the launch limit", m);
   }
-  GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmWorkspaceBytes(m, static_cast<uint32_t>(w->rows), nb)));
-  GUFO_HIP_TRY(gufo::LaunchGemm(w->type, w->data, static_cast<uint32_t>(w->rows), nb, a, m,
-                                g_state.gemm_work.ptr, c, g_state.stream));
+  // A prepared matrix brings its fragments; otherwise the workspace holds them for the
+  // duration of the call.
+  const size_t own_weights =
+      w->prefill_fragments != nullptr ? 0 : gufo::GemmWeightBytes(static_cast<uint32_t>(w->rows), nb);
+  GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmActivationBytes(m, nb) + own_weights));
+  GUFO_HIP_TRY(gufo::LaunchGemm(w->type, w->data, static_cast<uint32_t>(w->rows), nb,
+                                w->prefill_fragments, a, m, g_state.gemm_work.ptr, c,
+                                g_state.stream));
   return GUFO_HIP_OK;
 }
 

@@ -176,17 +176,26 @@ hipError_t LaunchMoeCombineDirect(const float* rows, const float* weights, const
 
 // ---- prefill ------------------------------------------------------------------
 
-// Bytes of device workspace LaunchGemm needs: both operands as fp16.
-size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row);
+// Both operands of the prefill product as fp16: bytes of the activations of `tokens`
+// rows, and of a matrix's weights as matrix-instruction fragments.
+size_t GemmActivationBytes(size_t tokens, uint32_t blocks_per_row);
+size_t GemmWeightBytes(uint32_t rows, uint32_t blocks_per_row);
 
 // Row types LaunchGemm takes: Q4_K, Q5_K, Q6_K, Q8_0.
 bool GemmTakesType(int type);
 
+// The weights of w as fragments (GemmWeightBytes), once, for every product that follows.
+hipError_t LaunchGemmPrepareWeights(int type, const uint8_t* w, uint32_t rows,
+                                    uint32_t blocks_per_row, void* fragments,
+                                    hipStream_t stream);
+
 // c[t*rows + r] = row r of the matrix w (rows of `type`) . a[t], a given as bf16
 // (tokens x blocks_per_row*256), on the matrix cores with fp32 accumulation.
+// `fragments`: what LaunchGemmPrepareWeights wrote for w, or null; `workspace` holds
+// GemmActivationBytes, plus GemmWeightBytes when fragments is null.
 hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
-                      const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
-                      hipStream_t stream);
+                      const void* fragments, const uint16_t* a_bf16, size_t tokens,
+                      void* workspace, float* c, hipStream_t stream);
 
 // index of the first maximum of v[0..n) -> *out (device); scratch holds
 // 2*kArgmaxBlocks entries of 8 bytes.

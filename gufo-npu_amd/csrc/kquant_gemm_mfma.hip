@@ -733,35 +733,19 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
 
 }  // namespace
 
-// Activations as fp16, then the fragments of every 32 rows of every row tile.
-size_t GemmWorkspaceBytes(size_t tokens, uint32_t rows, uint32_t blocks_per_row) {
-  const size_t act_bytes = (tokens * blocks_per_row * 512 + 255) & ~static_cast<size_t>(255);
-  const size_t row_tiles = (static_cast<size_t>(rows) + kTileRows - 1) / kTileRows;
-  return act_bytes + row_tiles * kTileGroups * blocks_per_row * 2 * kHalfBytes;
-}
+namespace {
 
-bool GemmTakesType(int type) {
-  return type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ80;
-}
-
-hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
-                      const uint16_t* a_bf16, size_t tokens, void* workspace, float* c,
-                      hipStream_t stream) {
-  if (!GemmTakesType(type)) return hipErrorInvalidValue;
-  if (rows == 0 || tokens == 0) return hipSuccess;
-  // Activation bytes are addressed with 32 bits.
-  if (blocks_per_row == 0 || tokens > 0xFFFFFFFFull / (512ull * blocks_per_row)) {
-    return hipErrorInvalidValue;
-  }
-  const size_t octets = tokens * blocks_per_row * 32;
-  const size_t act_bytes = (octets * 16 + 255) & ~static_cast<size_t>(255);
-  uint8_t* a16 = static_cast<uint8_t*>(workspace);
-  uint8_t* w16 = a16 + act_bytes;
+// The pre-pass over `octets` activation octets (none: a null `a_bf16`) and, when `w` is
+// given, over the weights.
+hipError_t LaunchPrepare(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
+                         const uint16_t* a_bf16, size_t octets, uint8_t* a16, uint8_t* w16,
+                         hipStream_t stream) {
   const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
   const uint32_t row_groups = row_tiles * kTileGroups;
-  const uint32_t act_groups = static_cast<uint32_t>((octets + 255) / 256);
+  const uint32_t act_groups = a_bf16 != nullptr ? static_cast<uint32_t>((octets + 255) / 256) : 0;
   // One workgroup (4 waves) per (32 rows, super-block): a wave per quarter.
-  const uint32_t weight_groups = row_groups * blocks_per_row;
+  const uint32_t weight_groups = w != nullptr ? row_groups * blocks_per_row : 0;
+  if (weight_groups + act_groups == 0) return hipSuccess;
   auto prepare = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(weight_groups + act_groups), dim3(256), 0, stream,
                        reinterpret_cast<const U32x4*>(a_bf16), octets,
@@ -774,7 +758,50 @@ hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks
     case kTypeQ6K: prepare(PrepareOperands<kTypeQ6K>); break;
     default: prepare(PrepareOperands<kTypeQ80>); break;
   }
-  hipError_t status = hipGetLastError();
+  return hipGetLastError();
+}
+
+}  // namespace
+
+size_t GemmActivationBytes(size_t tokens, uint32_t blocks_per_row) {
+  return (tokens * blocks_per_row * 512 + 255) & ~static_cast<size_t>(255);
+}
+
+// The fragments of every 32 rows of every row tile.
+size_t GemmWeightBytes(uint32_t rows, uint32_t blocks_per_row) {
+  const size_t row_tiles = (static_cast<size_t>(rows) + kTileRows - 1) / kTileRows;
+  return row_tiles * kTileGroups * blocks_per_row * 2 * kHalfBytes;
+}
+
+bool GemmTakesType(int type) {
+  return type == kTypeQ4K || type == kTypeQ5K || type == kTypeQ6K || type == kTypeQ80;
+}
+
+hipError_t LaunchGemmPrepareWeights(int type, const uint8_t* w, uint32_t rows,
+                                    uint32_t blocks_per_row, void* fragments,
+                                    hipStream_t stream) {
+  if (!GemmTakesType(type) || blocks_per_row == 0) return hipErrorInvalidValue;
+  if (rows == 0) return hipSuccess;
+  return LaunchPrepare(type, w, rows, blocks_per_row, nullptr, 0, nullptr,
+                       static_cast<uint8_t*>(fragments), stream);
+}
+
+hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
+                      const void* fragments, const uint16_t* a_bf16, size_t tokens,
+                      void* workspace, float* c, hipStream_t stream) {
+  if (!GemmTakesType(type)) return hipErrorInvalidValue;
+  if (rows == 0 || tokens == 0) return hipSuccess;
+  // Activation bytes are addressed with 32 bits.
+  if (blocks_per_row == 0 || tokens > 0xFFFFFFFFull / (512ull * blocks_per_row)) {
+    return hipErrorInvalidValue;
+  }
+  const size_t octets = tokens * blocks_per_row * 32;
+  uint8_t* a16 = static_cast<uint8_t*>(workspace);
+  uint8_t* own_w16 = a16 + GemmActivationBytes(tokens, blocks_per_row);
+  const uint8_t* w16 = fragments != nullptr ? static_cast<const uint8_t*>(fragments) : own_w16;
+  const uint32_t row_tiles = (rows + kTileRows - 1) / kTileRows;
+  hipError_t status = LaunchPrepare(type, fragments != nullptr ? nullptr : w, rows,
+                                    blocks_per_row, a_bf16, octets, a16, own_w16, stream);
   if (status != hipSuccess) return status;
 
   constexpr size_t lds_bytes = static_cast<size_t>(kStages) * kStageBytes;

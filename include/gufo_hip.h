@@ -270,7 +270,14 @@ int gufo_hip_gemm_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, si
                        float* c_host);
 int gufo_hip_gemm_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev, size_t m,
                            float* c_dev);
-/* The same, refusing any w that is not Q4_K (the type of the prefill configuration). */
+/* Keeps w's weights in the form the prefill product multiplies from (fp16, 512 bytes
+ * per 256 weights, beside the packed rows) from now until w is destroyed, so that every
+ * gufo_hip_gemm_* call on w converts only its activations: the counterpart of the NPU
+ * backend keeping each matrix resident in its own layout (src/npu/gemv.hpp:134-145).
+ * Results do not change by a bit.  Not while recording. */
+int gufo_hip_matrix_prepare_prefill(gufo_hip_matrix* w);
+/* gufo_hip_gemm_bf16 and _dev, refusing any w that is not Q4_K (the type of the prefill
+ * configuration). */
 int gufo_hip_gemm_q4k_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host,
                            size_t m, float* c_host);
 int gufo_hip_gemm_q4k_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,

@@ -139,6 +139,38 @@ def test_gemm_unit_activations_return_the_weights_other_types(hip, oracle, ggml_
     m.destroy()
 
 
+@pytest.mark.parametrize("ggml_type", [synth.Q4_K, synth.Q6_K])
+def test_gemm_with_prepared_weights_gives_the_same_bits(hip, ggml_type):
+    # gufo_hip_matrix_prepare_prefill keeps the converted weights with the matrix: every
+    # later product skips that half of the pre-pass and must not change by a bit, whatever
+    # the token count, and a row subset taken from a prepared matrix stands on its own.
+    say("gemm prepared", synth.TYPE_NAMES[ggml_type])
+    rows, cols = 300, 768
+    w = synth.matrix(ggml_type, rows, cols, 7300 + ggml_type)
+    m = hip.Matrix(ggml_type, w, rows, cols)
+    inputs = [bf16_activations(tokens, cols, 7310 + tokens)[0] for tokens in (1, 130, 257)]
+    before = [hip.gemm_bf16(m, bits) for bits in inputs]
+    m.prepare_prefill()
+    m.prepare_prefill()  # a second call changes nothing
+    for bits, want in zip(inputs, before):
+        assert bool(np.array_equal(hip.gemm_bf16(m, bits).view(np.uint32), want.view(np.uint32)))
+    picked = m.gather_rows(np.arange(10, 74))
+    got = hip.gemm_bf16(picked, inputs[1])
+    assert bool(np.array_equal(got.view(np.uint32), before[1][:, 10:74].view(np.uint32)))
+    picked.destroy()
+    # the GEMV entry points are untouched by it
+    x = synth.activations(2, cols, 5)
+    y = hip.gemv([hip.whole(m)], x, 2)
+    m.destroy()
+    again = hip.Matrix(ggml_type, w, rows, cols)
+    assert bool(np.array_equal(hip.gemv([hip.whole(again)], x, 2).view(np.uint32), y.view(np.uint32)))
+    again.destroy()
+    f = hip.Matrix(synth.F32, synth.matrix(synth.F32, 32, 256, 2), 32, 256)
+    with pytest.raises(hip.InvalidArgumentError):
+        f.prepare_prefill()
+    f.destroy()
+
+
 def test_gemm_q4k_entry_point_equals_the_general_one(hip):
     w = synth.kquant_matrix(synth.Q4_K, 96, 512, 5)
     m = hip.Matrix(synth.Q4_K, w, 96, 512)
