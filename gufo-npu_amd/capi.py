@@ -105,6 +105,7 @@ SIGNATURES = {
                                          _P, _P]),
     "gufo_hip_gemm_bf16": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_bf16_dev": (C.c_int, [_P, _P, _SZ, _P]),
+    "gufo_hip_gemm_bf16_parts_dev": (C.c_int, [_P, C.c_int, _P, _SZ, _P]),
     "gufo_hip_gemm_q4k_bf16": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_gemm_q4k_bf16_dev": (C.c_int, [_P, _P, _SZ, _P]),
     "gufo_hip_capture_begin": (C.c_int, []),
@@ -418,6 +419,15 @@ def gemm_bf16(w: Matrix, a_bf16: np.ndarray) -> np.ndarray:
     c = np.empty((m, w.rows), dtype=np.float32)
     _check(load_library().gufo_hip_gemm_bf16(C.c_void_p(w.handle), _ptr(a_bf16), m, _ptr(c)))
     return c
+
+
+def gemm_bf16_parts_dev(parts: Sequence[Matrix], a: DeviceBuffer, m: int,
+                        c: DeviceBuffer) -> None:
+    """The prefill product of a stage's matrices, outputs side by side per token
+    (gufo_hip_gemm_bf16_parts_dev)."""
+    handles = (C.c_void_p * len(parts))(*[p.handle for p in parts])
+    _check(load_library().gufo_hip_gemm_bf16_parts_dev(handles, len(parts), C.c_void_p(a.ptr), m,
+                                                       C.c_void_p(c.ptr)))
 
 
 def gemm_bf16_dev(w: Matrix, a: DeviceBuffer, m: int, c: DeviceBuffer) -> None:

@@ -1123,35 +1123,69 @@ int gufo_hip_moe_ffn(const gufo_hip_matrix* gate, const gufo_hip_matrix* up,
 
 namespace {
 
-int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* c,
-                  bool q4k_only) {
-  if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
-  if (q4k_only && w->type != GUFO_HIP_Q4_K) {
-    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
-                "this entry point takes Q4_K weights; this matrix has ggml type %d", w->type);
+// The matrices of one stage (whole, sharing their input) against m rows of activations:
+// c[t*stride + offset_p + r], stride = the sum of their rows - MatMul's layout with
+// tokens = m (src/models/qwen35/gguf_projections.cpp:239-286).
+int GemmPartsDevLocked(const gufo_hip_matrix* const* parts, int n_parts, const uint16_t* a,
+                       size_t m, float* c, bool q4k_only) {
+  if (parts == nullptr || n_parts < 1) {
+    return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
   }
-  if (!gufo::GemmTakesType(w->type)) {
-    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
-                "the prefill GEMM takes Q4_K, Q5_K, Q6_K or Q8_0 weights; this matrix has "
-                "ggml type %d",
-                w->type);
+  size_t stride = 0;
+  size_t own_weights = 0;
+  for (int p = 0; p < n_parts; ++p) {
+    const gufo_hip_matrix* w = parts[p];
+    if (w == nullptr) return Fail(GUFO_HIP_ERR_LOGIC, "no weights for this product");
+    if (q4k_only && w->type != GUFO_HIP_Q4_K) {
+      return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                  "this entry point takes Q4_K weights; this matrix has ggml type %d", w->type);
+    }
+    if (!gufo::GemmTakesType(w->type)) {
+      return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT,
+                  "the prefill GEMM takes Q4_K, Q5_K, Q6_K or Q8_0 weights; this matrix has "
+                  "ggml type %d",
+                  w->type);
+    }
+    if (w->cols != parts[0]->cols) {
+      return Fail(GUFO_HIP_ERR_SHAPE, "part %d has rows of %zu values, part 0 of %zu", p,
+                  w->cols, parts[0]->cols);
+    }
+    stride += w->rows;
+    // A prepared matrix brings its fragments; otherwise the workspace holds them for the
+    // duration of its product (one matrix after the other, so the largest decides).
+    if (w->prefill_fragments == nullptr) {
+      const size_t bytes = gufo::GemmWeightBytes(
+          static_cast<uint32_t>(w->rows), static_cast<uint32_t>(w->cols / gufo::kSuperBlock));
+      if (bytes > own_weights) own_weights = bytes;
+    }
   }
-  if (m == 0 || w->rows == 0) return GUFO_HIP_OK;
+  if (m == 0 || stride == 0) return GUFO_HIP_OK;
   if (a == nullptr || c == nullptr) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a or c is null");
   if (!Aligned16(a)) return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "a must be 16-byte aligned");
-  const uint32_t nb = static_cast<uint32_t>(w->cols / gufo::kSuperBlock);
-  if (m > (1ull << 24)) {
-    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens exceed the launch limit", m);
+  const uint32_t nb = static_cast<uint32_t>(parts[0]->cols / gufo::kSuperBlock);
+  if (m > (1ull << 24) || stride > 0xFFFFFFFFull) {
+    return Fail(GUFO_HIP_ERR_INVALID_ARGUMENT, "%zu tokens x %zu outputs exceed the launch limit",
+                m, stride);
   }
-  // A prepared matrix brings its fragments; otherwise the workspace holds them for the
-  // duration of the call.
-  const size_t own_weights =
-      w->prefill_fragments != nullptr ? 0 : gufo::GemmWeightBytes(static_cast<uint32_t>(w->rows), nb);
   GUFO_TRY(Reserve(&g_state.gemm_work, gufo::GemmActivationBytes(m, nb) + own_weights));
-  GUFO_HIP_TRY(gufo::LaunchGemm(w->type, w->data, static_cast<uint32_t>(w->rows), nb,
-                                w->prefill_fragments, a, m, g_state.gemm_work.ptr, c,
-                                g_state.stream));
+  size_t offset = 0;
+  bool converted = false;  // the activations are converted by the first launch
+  for (int p = 0; p < n_parts; ++p) {
+    const gufo_hip_matrix* w = parts[p];
+    if (w->rows == 0) continue;
+    GUFO_HIP_TRY(gufo::LaunchGemm(w->type, w->data, static_cast<uint32_t>(w->rows), nb,
+                                  w->prefill_fragments, converted ? nullptr : a, m,
+                                  g_state.gemm_work.ptr, c + offset,
+                                  static_cast<uint32_t>(stride), g_state.stream));
+    converted = true;
+    offset += w->rows;
+  }
   return GUFO_HIP_OK;
+}
+
+int GemmDevLocked(const gufo_hip_matrix* w, const uint16_t* a, size_t m, float* c,
+                  bool q4k_only) {
+  return GemmPartsDevLocked(&w, 1, a, m, c, q4k_only);
 }
 
 int GemmHostLocked(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,
@@ -1177,6 +1211,13 @@ int gufo_hip_gemm_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev,
   const std::lock_guard<std::mutex> lock(g_state.mutex);
   GUFO_TRY(RequireReady());
   return GemmDevLocked(w, a_bf16_dev, m, c_dev, false);
+}
+
+int gufo_hip_gemm_bf16_parts_dev(const gufo_hip_matrix* const* parts, int n_parts,
+                                 const uint16_t* a_bf16_dev, size_t m, float* c_dev) {
+  const std::lock_guard<std::mutex> lock(g_state.mutex);
+  GUFO_TRY(RequireReady());
+  return GemmPartsDevLocked(parts, n_parts, a_bf16_dev, m, c_dev, false);
 }
 
 int gufo_hip_gemm_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, size_t m,

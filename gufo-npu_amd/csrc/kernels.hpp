@@ -189,13 +189,15 @@ hipError_t LaunchGemmPrepareWeights(int type, const uint8_t* w, uint32_t rows,
                                     uint32_t blocks_per_row, void* fragments,
                                     hipStream_t stream);
 
-// c[t*rows + r] = row r of the matrix w (rows of `type`) . a[t], a given as bf16
+// c[t*c_stride + r] = row r of the matrix w (rows of `type`) . a[t], a given as bf16
 // (tokens x blocks_per_row*256), on the matrix cores with fp32 accumulation.
 // `fragments`: what LaunchGemmPrepareWeights wrote for w, or null; `workspace` holds
-// GemmActivationBytes, plus GemmWeightBytes when fragments is null.
+// GemmActivationBytes, plus GemmWeightBytes when fragments is null.  A null a_bf16 means
+// the workspace still holds the converted activations of the call before (the next
+// matrix of a stage, which shares its input).
 hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
                       const void* fragments, const uint16_t* a_bf16, size_t tokens,
-                      void* workspace, float* c, hipStream_t stream);
+                      void* workspace, float* c, uint32_t c_stride, hipStream_t stream);
 
 // index of the first maximum of v[0..n) -> *out (device); scratch holds
 // 2*kArgmaxBlocks entries of 8 bytes.

@@ -396,6 +396,7 @@ __device__ __forceinline__ constexpr uint32_t StepPiece(int s) {
 
 struct GemmShape {
   uint32_t rows;
+  uint32_t c_stride;     // floats between the token rows of c
   uint32_t nb;           // super-blocks per row
   uint32_t tokens;
   uint32_t row_tiles;
@@ -667,12 +668,12 @@ KquantGemmKernel(const uint8_t* __restrict__ w16, const uint8_t* __restrict__ a1
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
           const uint32_t t0 = token_first + m * 32 + 4 * u;
-          float* at = c + static_cast<size_t>(t0) * shape.rows + row;
+          float* at = c + static_cast<size_t>(t0) * shape.c_stride + row;
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const uint32_t dt = 8 * (i >> 2) + (i & 3);
             if (!decltype(check)::value || (t0 + dt < shape.tokens && row < shape.rows)) {
-              at[static_cast<size_t>(dt) * shape.rows] = acc[g][m][i];
+              at[static_cast<size_t>(dt) * shape.c_stride] = acc[g][m][i];
             }
           }
         }
@@ -788,8 +789,8 @@ hipError_t LaunchGemmPrepareWeights(int type, const uint8_t* w, uint32_t rows,
 
 hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks_per_row,
                       const void* fragments, const uint16_t* a_bf16, size_t tokens,
-                      void* workspace, float* c, hipStream_t stream) {
-  if (!GemmTakesType(type)) return hipErrorInvalidValue;
+                      void* workspace, float* c, uint32_t c_stride, hipStream_t stream) {
+  if (!GemmTakesType(type) || c_stride < rows) return hipErrorInvalidValue;
   if (rows == 0 || tokens == 0) return hipSuccess;
   // Activation bytes are addressed with 32 bits.
   if (blocks_per_row == 0 || tokens > 0xFFFFFFFFull / (512ull * blocks_per_row)) {
@@ -815,6 +816,7 @@ hipError_t LaunchGemm(int type, const uint8_t* w, uint32_t rows, uint32_t blocks
   }
   GemmShape shape;
   shape.rows = rows;
+  shape.c_stride = c_stride;
   shape.nb = blocks_per_row;
   shape.tokens = static_cast<uint32_t>(tokens);
   shape.row_tiles = row_tiles;

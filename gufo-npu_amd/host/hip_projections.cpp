@@ -237,6 +237,26 @@ void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, 
                                 whole.count(), &prologue, in.x, tokens, y));
 }
 
+void HipProjections::PrefillDevice(Stage stage, int layer, const std::uint16_t* a_bf16,
+                                   std::size_t tokens, float* c) const {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  if (parts == nullptr || parts->empty()) {
+    throw std::logic_error("qwen35: no weights for this stage and layer");
+  }
+  std::vector<const gufo_hip_matrix*> handles;
+  for (const Matrix& m : *parts) handles.push_back(m.handle);
+  Check(gufo_hip_gemm_bf16_parts_dev(handles.data(), static_cast<int>(handles.size()), a_bf16,
+                                     tokens, c));
+}
+
+void HipProjections::PreparePrefill(Stage stage, int layer) {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  if (parts == nullptr || parts->empty()) {
+    throw std::logic_error("qwen35: no weights for this stage and layer");
+  }
+  for (const Matrix& m : *parts) Check(gufo_hip_matrix_prepare_prefill(m.handle));
+}
+
 void HipProjections::PickDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
                                 std::int64_t* index) const {
   const std::vector<Matrix>* parts = StageMatrices(stage, layer);

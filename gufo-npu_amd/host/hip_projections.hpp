@@ -137,6 +137,17 @@ public:
   void PickDevice(Stage stage, int layer, const DeviceInput& in, int tokens,
                   std::int64_t* index) const;
 
+  // A stage for many tokens at once on the matrix cores, the prefill shape: a_bf16
+  // (device, tokens x stage input, bf16 as the reference's NPU prefill GEMM takes its
+  // activations, src/npu/gemm.hpp:99-105), c (device) tokens x stage output fp32 in
+  // Apply's layout.  Quantized row types only; held to 1e-3 relative, not Apply's 1e-4
+  // (fp16 operands).  Enqueued, not waited for.
+  void PrefillDevice(Stage stage, int layer, const std::uint16_t* a_bf16, std::size_t tokens,
+                     float* c) const;
+  // Keeps the stage's weights in PrefillDevice's own form as well (3.5 x their packed
+  // size) so that later calls convert only their activations.
+  void PreparePrefill(Stage stage, int layer);
+
   // qwen35::Route (src/models/qwen35/moe.cpp:16-42) on the device.
   void Route(const float* logits, int tokens, int k, int* chosen, float* weights) const;
   // The routed experts of one MoE layer in one call: what Decoder::MoeFfn /

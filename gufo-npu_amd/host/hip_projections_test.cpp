@@ -474,6 +474,51 @@ void RunPick(std::mt19937& rng) {
   }
 }
 
+// A stage for many tokens on the matrix cores: PrefillDevice against Apply on the same
+// (bf16-representable) activations, before and after PreparePrefill.
+void RunPrefill(std::mt19937& rng) {
+  const std::size_t hidden = 512, ffn = 320, tokens = 70;
+  const Weights gate = RandomWeights(GUFO_ORACLE_Q4_K, ffn, hidden, rng);
+  const Weights up = RandomWeights(GUFO_ORACLE_Q5_K, ffn, hidden, rng);
+  ModelTensors model;
+  model.hidden = static_cast<int>(hidden);
+  LayerTensors layer;
+  layer.ffn_in = {AsTensor("blk.0.ffn_gate.weight", gate), AsTensor("blk.0.ffn_up.weight", up)};
+  model.layers.push_back(layer);
+  HipProjections proj(model);
+
+  auto x = RandomActivations(tokens * hidden, rng);
+  std::vector<std::uint16_t> bits(x.size());
+  for (std::size_t i = 0; i < x.size(); ++i) {  // round to bf16, nearest even
+    std::uint32_t u;
+    std::memcpy(&u, &x[i], 4);
+    u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+    std::memcpy(&x[i], &u, 4);
+    bits[i] = static_cast<std::uint16_t>(u >> 16);
+  }
+  std::vector<float> want(tokens * 2 * ffn);
+  proj.Apply(Stage::kFfnIn, 0, x.data(), static_cast<int>(tokens), want.data());
+
+  void* d_bits = nullptr;
+  if (gufo_hip_malloc(&d_bits, bits.size() * 2) != GUFO_HIP_OK) throw std::bad_alloc();
+  gufo_hip_memcpy_h2d(d_bits, bits.data(), bits.size() * 2);
+  const DeviceRows d_c(want.size());
+  proj.PrefillDevice(Stage::kFfnIn, 0, static_cast<const std::uint16_t*>(d_bits), tokens,
+                     d_c.get());
+  const auto first = d_c.Download();
+  double err = RelL2(first, want);
+  Report("PrefillDevice kFfnIn equals Apply within 1e-3", err <= 1e-3, err);
+  proj.PreparePrefill(Stage::kFfnIn, 0);
+  proj.PrefillDevice(Stage::kFfnIn, 0, static_cast<const std::uint16_t*>(d_bits), tokens,
+                     d_c.get());
+  Report("PrefillDevice after PreparePrefill: the same bits", d_c.Download() == first);
+  Report("PrefillDevice on a missing stage throws std::logic_error", Throws<std::logic_error>([&] {
+           proj.PrefillDevice(Stage::kFfnDown, 0, static_cast<const std::uint16_t*>(d_bits),
+                              tokens, d_c.get());
+         }));
+  gufo_hip_free(d_bits);
+}
+
 // Decoder::MoeFfn in one call on device rows (src/models/qwen35/decoder.cpp:530-558)
 // against the same steps through the host-pointer methods: the kRouter product (two
 // tensors: the experts' rows and the shared expert's gate row), Route, RoutedFfn, and the
@@ -540,6 +585,7 @@ int main(int argc, char** argv) {
     RunDense(rng);
     RunMoe(rng);
     RunMoeLayer(rng);
+    RunPrefill(rng);
     RunDeviceChain(rng);
     RunPick(rng);
   } catch (const std::exception& e) {

@@ -270,6 +270,12 @@ int gufo_hip_gemm_bf16(const gufo_hip_matrix* w, const uint16_t* a_bf16_host, si
                        float* c_host);
 int gufo_hip_gemm_bf16_dev(const gufo_hip_matrix* w, const uint16_t* a_bf16_dev, size_t m,
                            float* c_dev);
+/* The same for the matrices of one stage (whole, sharing their input), their outputs side
+ * by side within a token's row as MatMul lays them out (gguf_projections.cpp:264-283):
+ *   c[t*stride + offset_p + r] = row r of parts[p] . a[t],  stride = the sum of the rows.
+ * The activations are converted once for all parts. */
+int gufo_hip_gemm_bf16_parts_dev(const gufo_hip_matrix* const* parts, int n_parts,
+                                 const uint16_t* a_bf16_dev, size_t m, float* c_dev);
 /* Keeps w's weights in the form the prefill product multiplies from (fp16, 512 bytes
  * per 256 weights, beside the packed rows) from now until w is destroyed, so that every
  * gufo_hip_gemm_* call on w converts only its activations: the counterpart of the NPU

@@ -171,6 +171,39 @@ def test_gemm_with_prepared_weights_gives_the_same_bits(hip, ggml_type):
     f.destroy()
 
 
+def test_gemm_of_a_stage_lays_its_parts_side_by_side(hip, oracle):
+    # [q | k | v]-like: three matrices of two types sharing their input, one of them with
+    # prepared weights; c[t] = [part 0 | part 1 | part 2], each column block bit for bit
+    # the matrix's own product, ragged row counts included.
+    say("gemm parts")
+    cols, tokens = 512, 150
+    shapes = [(synth.Q4_K, 200), (synth.Q6_K, 33), (synth.Q4_K, 64)]
+    blocks = [synth.matrix(t, rows, cols, 7400 + i) for i, (t, rows) in enumerate(shapes)]
+    mats = [hip.Matrix(t, b, rows, cols) for (t, rows), b in zip(shapes, blocks)]
+    mats[2].prepare_prefill()
+    bits, a = bf16_activations(tokens, cols, 7410)
+    stride = sum(rows for _, rows in shapes)
+    da = hip.DeviceBuffer.from_array(bits)
+    dc = hip.DeviceBuffer(4 * tokens * stride)
+    hip.gemm_bf16_parts_dev(mats, da, tokens, dc)
+    hip.synchronize()
+    got = dc.download((tokens, stride), np.float32)
+    offset = 0
+    for m, (_, rows) in zip(mats, shapes):
+        alone = hip.gemm_bf16(m, bits)
+        assert bool(np.array_equal(got[:, offset:offset + rows].view(np.uint32),
+                                   alone.view(np.uint32)))
+        offset += rows
+    want = oracle.matmul([(t, b, 0, rows) for (t, rows), b in zip(shapes, blocks)], a,
+                         precision="double", threads=8)
+    assert oracle.rel_l2(got, want) <= TOLERANCE
+    other = hip.Matrix(synth.Q4_K, synth.matrix(synth.Q4_K, 32, 256, 1), 32, 256)
+    with pytest.raises(hip.ShapeError):
+        hip.gemm_bf16_parts_dev([mats[0], other], da, tokens, dc)
+    for m in mats + [other]:
+        m.destroy()
+
+
 def test_gemm_q4k_entry_point_equals_the_general_one(hip):
     w = synth.kquant_matrix(synth.Q4_K, 96, 512, 5)
     m = hip.Matrix(synth.Q4_K, w, 96, 512)
