@@ -237,6 +237,24 @@ void HipProjections::ApplyDevice(Stage stage, int layer, const DeviceInput& in, 
                                 whole.count(), &prologue, in.x, tokens, y));
 }
 
+std::vector<const gufo_hip_matrix*> HipProjections::StageHandles(Stage stage, int layer) const {
+  const std::vector<Matrix>* parts = StageMatrices(stage, layer);
+  std::vector<const gufo_hip_matrix*> handles;
+  if (parts != nullptr) {
+    for (const Matrix& m : *parts) handles.push_back(m.handle);
+  }
+  return handles;
+}
+
+void HipProjections::ExpertHandles(int layer, const gufo_hip_matrix** gate,
+                                   const gufo_hip_matrix** up,
+                                   const gufo_hip_matrix** down) const {
+  const Layer& l = layers_.at(static_cast<std::size_t>(layer));
+  if (gate != nullptr) *gate = l.gate_exps.handle;
+  if (up != nullptr) *up = l.up_exps.handle;
+  if (down != nullptr) *down = l.down_exps.handle;
+}
+
 void HipProjections::PrefillDevice(Stage stage, int layer, const std::uint16_t* a_bf16,
                                    std::size_t tokens, float* c) const {
   const std::vector<Matrix>* parts = StageMatrices(stage, layer);

@@ -148,6 +148,13 @@ public:
   // size) so that later calls convert only their activations.
   void PreparePrefill(Stage stage, int layer);
 
+  // The resident matrices of a stage, in the order of its parts, and the three expert
+  // tensors of a mixture layer (gate, up, down; null for a dense layer): for callers that
+  // drive the C entry points of gufo_hip.h themselves.  They belong to this object.
+  std::vector<const gufo_hip_matrix*> StageHandles(Stage stage, int layer) const;
+  void ExpertHandles(int layer, const gufo_hip_matrix** gate, const gufo_hip_matrix** up,
+                     const gufo_hip_matrix** down) const;
+
   // qwen35::Route (src/models/qwen35/moe.cpp:16-42) on the device.
   void Route(const float* logits, int tokens, int k, int* chosen, float* weights) const;
   // The routed experts of one MoE layer in one call: what Decoder::MoeFfn /

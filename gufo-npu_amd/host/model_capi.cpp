@@ -157,6 +157,30 @@ int gufo_model_apply_expert(const gufo_model* model, int stage, int layer, int e
   });
 }
 
+int gufo_model_stage_matrices(const gufo_model* model, int stage, int layer,
+                              const gufo_hip_matrix** out, int capacity, int* count) {
+  return Guarded([&] {
+    RequireModel(model);
+    if (count == nullptr) throw std::invalid_argument("count is null");
+    const auto handles = model->impl.projections().StageHandles(StageOf(stage), layer);
+    *count = static_cast<int>(handles.size());
+    if (out == nullptr) return;
+    if (capacity < *count) {
+      throw std::invalid_argument("room for " + std::to_string(capacity) + " of " +
+                                  std::to_string(*count) + " matrices");
+    }
+    std::copy(handles.begin(), handles.end(), out);
+  });
+}
+
+int gufo_model_expert_matrices(const gufo_model* model, int layer, const gufo_hip_matrix** gate,
+                               const gufo_hip_matrix** up, const gufo_hip_matrix** down) {
+  return Guarded([&] {
+    RequireModel(model);
+    model->impl.projections().ExpertHandles(layer, gate, up, down);
+  });
+}
+
 int gufo_model_norm_weight(const gufo_model* model, int which, int layer, float* out) {
   return Guarded([&] {
     RequireModel(model);

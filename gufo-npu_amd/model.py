@@ -35,6 +35,21 @@ class Shape(C.Structure):
         return {name: getattr(self, name) for name, _ in self._fields_}
 
 
+class BorrowedMatrix(capi.Matrix):
+    """A resident matrix that belongs to an open model: usable wherever a capi.Matrix is,
+    never destroyed from here."""
+
+    def __init__(self, handle):
+        self.handle = handle
+        self.type, self.rows, self.cols, self.nbytes = self.info()
+
+    def destroy(self) -> None:
+        self.handle = None
+
+    def __del__(self):
+        pass
+
+
 _P = C.c_void_p
 # name -> (restype, argtypes): every symbol include/gufo_hip_model.h declares.
 SIGNATURES = {
@@ -46,6 +61,10 @@ SIGNATURES = {
     "gufo_model_weight_bytes": (C.c_uint64, [_P]),
     "gufo_model_stage_inputs": (C.c_size_t, [_P, C.c_int, C.c_int]),
     "gufo_model_stage_outputs": (C.c_size_t, [_P, C.c_int, C.c_int]),
+    "gufo_model_stage_matrices": (C.c_int, [_P, C.c_int, C.c_int, _P, C.c_int,
+                                            C.POINTER(C.c_int)]),
+    "gufo_model_expert_matrices": (C.c_int, [_P, C.c_int, C.POINTER(_P), C.POINTER(_P),
+                                             C.POINTER(_P)]),
     "gufo_model_apply": (C.c_int, [_P, C.c_int, C.c_int, _P, C.c_int, _P]),
     "gufo_model_apply_expert": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, _P, C.c_int, _P]),
     "gufo_model_norm_weight": (C.c_int, [_P, C.c_int, C.c_int, _P]),
@@ -105,6 +124,28 @@ class Model:
 
     def stage_outputs(self, stage: int, layer: int) -> int:
         return int(load_library().gufo_model_stage_outputs(self.handle, stage, layer))
+
+    @staticmethod
+    def _borrowed(handle) -> "BorrowedMatrix | None":
+        return BorrowedMatrix(handle) if handle else None
+
+    def stage_matrices(self, stage: int, layer: int) -> list:
+        """The resident matrices of a stage (gufo_model_stage_matrices), usable with
+        capi's device entry points for as long as the model is open."""
+        count = C.c_int()
+        _check(load_library().gufo_model_stage_matrices(self.handle, stage, layer, None, 0,
+                                                        C.byref(count)))
+        handles = (_P * max(count.value, 1))()
+        _check(load_library().gufo_model_stage_matrices(self.handle, stage, layer, handles,
+                                                        count.value, C.byref(count)))
+        return [self._borrowed(handles[i]) for i in range(count.value)]
+
+    def expert_matrices(self, layer: int):
+        """gate, up, down expert tensors of a mixture layer (None each for a dense one)."""
+        gate, up, down = _P(), _P(), _P()
+        _check(load_library().gufo_model_expert_matrices(self.handle, layer, C.byref(gate),
+                                                         C.byref(up), C.byref(down)))
+        return tuple(self._borrowed(h.value) for h in (gate, up, down))
 
     def apply(self, stage: int, layer: int, x: np.ndarray, expert: int = -1) -> np.ndarray:
         """Projections::Apply (ApplyExpert with expert >= 0) on tokens x inputs rows."""

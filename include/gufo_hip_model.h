@@ -93,6 +93,22 @@ uint64_t gufo_model_weight_bytes(const gufo_model* model);
 size_t gufo_model_stage_inputs(const gufo_model* model, int stage, int layer);
 size_t gufo_model_stage_outputs(const gufo_model* model, int stage, int layer);
 
+/* The resident matrices behind a stage, in the order of its parts
+ * (src/models/qwen35/gguf_projections.cpp:100-175), for callers that keep their rows on
+ * the device and drive gufo_hip.h's "_dev" entry points themselves (gufo_hip_gemv_fused_dev,
+ * gufo_hip_gemv_argmax_dev, gufo_hip_gemm_bf16_parts_dev, gufo_hip_moe_layer_dev ...).
+ * *count receives the number of parts (0 for a stage the layer does not have); with `out`
+ * given, `capacity` must hold them.  The handles belong to the model: never destroy them. */
+struct gufo_hip_matrix;
+int gufo_model_stage_matrices(const gufo_model* model, int stage, int layer,
+                              const struct gufo_hip_matrix** out, int capacity, int* count);
+/* The expert tensors of a mixture layer (ffn_gate_exps, ffn_up_exps, ffn_down_exps); null
+ * for a dense layer.  Any of the three pointers may be null. */
+int gufo_model_expert_matrices(const gufo_model* model, int layer,
+                               const struct gufo_hip_matrix** gate,
+                               const struct gufo_hip_matrix** up,
+                               const struct gufo_hip_matrix** down);
+
 /* Projections::Apply: y[t] = W x[t], host pointers, any tokens >= 0.  `layer` is ignored
  * for GUFO_STAGE_LM_HEAD. */
 int gufo_model_apply(const gufo_model* model, int stage, int layer, const float* x,

@@ -119,3 +119,64 @@ def test_calls_the_reference_refuses(opened):
             model.apply(hip_model.EXPERT_IN, 0, x, expert=0)
     with pytest.raises(capi.InvalidArgumentError):
         model.apply(42, 0, x)
+
+
+def test_a_loaded_model_lends_its_matrices_to_the_device_entry_points(opened, hip, oracle):
+    # gufo_model_stage_matrices / _expert_matrices: the matrices a model file was loaded
+    # into, used with rows that stay on the device.  Apply through the handles equals
+    # Apply through the model bit for bit; the stages with a prologue, the prefill product
+    # and - on the mixture model - the whole mixture layer run on them.
+    name, spec, golden, model = opened
+    from gufo_npu_amd import synth
+    hidden, tokens = model.shape["hidden"], 3
+    x = synth.activations(tokens, hidden, 4242) * np.float32(0.1)
+    dx = hip.DeviceBuffer.from_array(x)
+    for stage in (hip_model.ATTENTION_IN, hip_model.FFN_IN, hip_model.LM_HEAD):
+        layer = -1 if stage == hip_model.LM_HEAD else 0
+        mats = model.stage_matrices(stage, layer)
+        if not mats:  # a stage this layer does not have
+            assert model.stage_outputs(stage, layer) == 0
+            continue
+        say(name, "borrowed", hip_model.STAGE_NAMES[stage], len(mats), "matrices")
+        outputs = model.stage_outputs(stage, layer)
+        assert sum(m.rows for m in mats) == outputs and all(m.cols == hidden for m in mats)
+        dy = hip.DeviceBuffer(4 * tokens * outputs)
+        hip.gemv_dev([hip.whole(m) for m in mats], dx, tokens, dy)
+        hip.synchronize()
+        got = dy.download((tokens, outputs), np.float32)
+        want = model.apply(stage, layer, x)
+        assert bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
+        if all(m.type in (synth.Q4_K, synth.Q5_K, synth.Q6_K, synth.Q8_0) for m in mats):
+            bits = synth.bf16_round(x)
+            da = hip.DeviceBuffer.from_array(bits)
+            hip.gemm_bf16_parts_dev(mats, da, tokens, dy)
+            hip.synchronize()
+            prefill = dy.download((tokens, outputs), np.float32)
+            assert oracle.rel_l2(prefill, model.apply(stage, layer, synth.bf16_to_float(bits))) <= 1e-3
+    assert model.stage_matrices(hip_model.MTP_IN, 0) == [] or spec.mtp_layers > 0
+    gate, up, down = model.expert_matrices(0)
+    if not model.shape["is_moe"]:
+        assert gate is None and up is None and down is None
+        return
+    experts, k = model.shape["experts"], model.shape["experts_used"]
+    router = model.stage_matrices(hip_model.ROUTER, 0)
+    say(name, "mixture layer on borrowed matrices:", len(router), "router tensors")
+    shared = synth.activations(tokens, hidden, 4243)
+    ds = hip.DeviceBuffer.from_array(shared)
+    dy = hip.DeviceBuffer(4 * tokens * hidden)
+    hip.moe_layer_dev(router, gate, up, down, experts, k, dx, tokens, ds, dy)
+    hip.synchronize()
+    got = dy.download((tokens, hidden), np.float32)
+    # the same through the model's host-pointer calls, as Decoder::MoeFfn makes them
+    logits = model.apply(hip_model.ROUTER, 0, x)
+    assert logits.shape[1] == experts + 1
+    ids, weights = hip.route_topk(np.ascontiguousarray(logits[:, :experts]), k)
+    want = np.zeros((tokens, hidden), np.float64)
+    for t in range(tokens):
+        want[t] = shared[t] * oracle.shared_expert_scale(logits[t, experts])
+        for slot in range(k):
+            e = int(ids[t, slot])
+            gu = model.apply(hip_model.EXPERT_IN, 0, x[t:t + 1], e)
+            act = oracle.swiglu(gu)
+            want[t] += np.float64(weights[t, slot]) * model.apply(hip_model.EXPERT_DOWN, 0, act, e)[0]
+    assert oracle.rel_l2(got, want) <= 1e-5
